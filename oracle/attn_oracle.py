@@ -1,0 +1,340 @@
+"""CPU oracle for the attention hot path (TEST INFRASTRUCTURE, not product code).
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module, and only as the checker. The product path
+(the HIP library behind ``include/mi355_attn.h``) never calls into it.
+
+What is restated from the reference tree (paths relative to the reference root):
+
+* ``init_attention_mask`` / ``fill_attention_mask`` follow
+  ``runtime/executor/litert_compiled_model_executor_utils.cc:332-397``.
+* ``prefill_work_groups`` follows
+  ``runtime/executor/litert_compiled_model_executor_utils.cc:300-330``.
+* ``softmax_rows`` follows the max-subtracted form of
+  ``runtime/components/sampling_cpu_util.cc:66-134`` and is pinned by the
+  known-answer values of ``runtime/components/sampling_cpu_util_test.cc:32-97``.
+* ``quantize_kv_int8`` / ``dequantize_kv_int8`` use the symmetric round/clamp
+  idiom of ``runtime/executor/llm_litert_npu_compiled_model_executor.cc:116-171``
+  with a per-(kv head, channel) scale.
+* ``OracleExecutor`` restates the step / position / deferred-last-token
+  bookkeeping of ``runtime/executor/llm_litert_compiled_model_executor.cc:157-276``
+  (prefill), ``:416-534`` (decode), ``:568-574`` (reset) and
+  ``llm_litert_compiled_model_executor.h:95-97`` (current step).
+
+What is NOT in the reference tree: the attention arithmetic itself runs inside
+``litert::CompiledModel::Run`` (``llm_litert_compiled_model_executor.cc:271,407,522``),
+i.e. in LiteRT @c8f55dfb / TFLite+XNNPACK @734f7085, which are un-vendored
+``http_archive`` dependencies (``WORKSPACE:6-9,73-78,261-270``), executing a
+``.tflite`` graph that is absent too. ``sdpa_masked`` therefore restates the
+published scaled-dot-product-attention definition in the op order the in-tree
+call sites imply (additive float mask fed to the graph): scale -> QK^T -> +mask
+-> softmax -> PV, with GQA by KV-head broadcast. It is pinned by closed forms,
+invariants, brute force and a library cross-check (tests/test_oracle_*.py).
+
+PARITY UNPINNED (nothing in the reference tree or its fixtures fixes these; the
+choices below are the specification this build works to):
+  * bit-level fp32 results of XNNPACK's batch-matmul / softmax;
+  * the sliding-window boundary of local layers: here key j is visible to the
+    query at absolute position p iff ``0 <= p - j < window`` (self plus the
+    ``window - 1`` previous tokens);
+  * logit soft-capping form: ``cap * tanh(s / cap)`` applied after scaling.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+# Masked-out value of a float mask when the calculation precision is f16, and
+# the full-precision variant (litert_compiled_model_executor_utils.cc:350-352).
+MASK_NEG_F16 = -45824.0
+MASK_NEG_F32 = -0.7 * float(np.finfo(np.float32).max)
+
+
+# --------------------------------------------------------------------------
+# Mask construction (reference: utils.cc:332-397)
+# --------------------------------------------------------------------------
+def init_attention_mask(rows: int, ctx: int, boolean: bool = False, is_f16: bool = True) -> np.ndarray:
+    """A fresh ``[1,1,rows,ctx]`` mask with every entry masked out."""
+    if boolean:
+        return np.zeros((1, 1, rows, ctx), dtype=np.bool_)
+    fill = MASK_NEG_F16 if is_f16 else MASK_NEG_F32
+    return np.full((1, 1, rows, ctx), fill, dtype=np.float32)
+
+
+def fill_attention_mask(mask: np.ndarray, start_timestep: int, steps: int) -> np.ndarray:
+    """Row i (< steps) opens keys ``0 .. start_timestep + i`` inclusive; rows
+    beyond ``steps`` stay fully masked. Works in place and returns the mask."""
+    if mask.ndim != 4:
+        raise ValueError("Attention mask must be 4D.")
+    ctx = mask.shape[3]
+    flat = mask.reshape(-1)
+    opened = True if mask.dtype == np.bool_ else 0.0
+    for i in range(steps):
+        step = start_timestep + i
+        flat[i * ctx: i * ctx + step + 1] = opened
+    return mask
+
+
+def visibility(q_pos: np.ndarray, n_keys: int, window: int = 0) -> np.ndarray:
+    """Boolean ``[len(q_pos), n_keys]``: key j visible to the query at absolute
+    position p iff j <= p (the causal rule of fill_attention_mask) and, on a
+    sliding-window layer, p - j < window."""
+    p = np.asarray(q_pos, dtype=np.int64)[:, None]
+    j = np.arange(n_keys, dtype=np.int64)[None, :]
+    vis = j <= p
+    if window and window > 0:
+        vis &= (p - j) < window
+    return vis
+
+
+# --------------------------------------------------------------------------
+# Softmax (reference style: sampling_cpu_util.cc:94-131)
+# --------------------------------------------------------------------------
+def softmax_rows(x: np.ndarray, temperature: float = 1.0, dtype=np.float64) -> np.ndarray:
+    """Max-subtracted softmax along the last axis."""
+    if temperature <= 0.0:
+        raise ValueError("Temperature must be positive")
+    x = np.asarray(x, dtype=dtype)
+    t = max(dtype(temperature), np.finfo(np.float32).eps)
+    m = x.max(axis=-1, keepdims=True)
+    e = np.exp((x - m) / t)
+    s = e.sum(axis=-1, keepdims=True)
+    return e / s
+
+
+# --------------------------------------------------------------------------
+# Scaled dot-product attention
+# --------------------------------------------------------------------------
+def _expand_kv(x: np.ndarray, n_q_heads: int) -> np.ndarray:
+    """[L, Hkv, D] -> [L, Hq, D] by KV-head broadcast: kv = q_head // (Hq/Hkv)."""
+    hkv = x.shape[1]
+    if n_q_heads % hkv:
+        raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+    return np.repeat(x, n_q_heads // hkv, axis=1)
+
+
+def sdpa_masked(q, k, v, scale: float, mask, softcap: float = 0.0, dtype=np.float64) -> np.ndarray:
+    """Attention with an explicit mask, in the op order scale -> QK^T -> +mask ->
+    softmax -> PV.
+
+    q ``[S, Hq, D]``, k/v ``[L, Hkv, D]``; mask ``[S, L]`` additive float or
+    boolean (True = visible). Returns ``[S, Hq, D]`` in ``dtype``.
+    """
+    q = np.asarray(q, dtype=dtype)
+    hq = q.shape[1]
+    kk = _expand_kv(np.asarray(k, dtype=dtype), hq)
+    vv = _expand_kv(np.asarray(v, dtype=dtype), hq)
+    s = np.einsum("shd,lhd->hsl", q * dtype(scale), kk)
+    if softcap and softcap > 0.0:
+        s = dtype(softcap) * np.tanh(s / dtype(softcap))
+    mask = np.asarray(mask)
+    if mask.dtype == np.bool_:
+        s = np.where(mask[None, :, :], s, -np.inf)
+    else:
+        s = s + mask.astype(dtype)[None, :, :]
+    m = s.max(axis=-1, keepdims=True)
+    m = np.where(np.isfinite(m), m, 0.0)
+    e = np.exp(s - m)
+    den = e.sum(axis=-1, keepdims=True)
+    # A row with no visible key (possible only for padded rows) yields zeros.
+    p = np.divide(e, den, out=np.zeros_like(e), where=den > 0)
+    return np.einsum("hsl,lhd->shd", p, vv)
+
+
+def sdpa(q, k, v, scale: float, q_pos0: int = 0, window: int = 0, softcap: float = 0.0,
+         kv_len: int | None = None, dtype=np.float64) -> np.ndarray:
+    """Causal (optionally sliding-window) attention by predicate.
+
+    Query row i sits at absolute position ``q_pos0 + i``; only the first
+    ``kv_len`` cache rows exist (default: all of k).
+    """
+    n = q.shape[0]
+    kv_len = k.shape[0] if kv_len is None else kv_len
+    vis = visibility(q_pos0 + np.arange(n), kv_len, window)
+    return sdpa_masked(q, k[:kv_len], v[:kv_len], scale, vis, softcap, dtype)
+
+
+def decode_attn(q, k, v, scale: float, kv_len: int, window: int = 0, softcap: float = 0.0,
+                dtype=np.float64) -> np.ndarray:
+    """One new token: q ``[Hq, D]`` at position ``kv_len - 1`` over a cache that
+    already holds that token's K/V row. Returns ``[Hq, D]``."""
+    return sdpa(q[None], k, v, scale, q_pos0=kv_len - 1, window=window, softcap=softcap,
+                kv_len=kv_len, dtype=dtype)[0]
+
+
+def decode_attn_split(q, k, v, scale: float, kv_len: int, num_splits: int, window: int = 0,
+                      softcap: float = 0.0, dtype=np.float64):
+    """Flash-decoding: the key range is cut into ``num_splits`` contiguous
+    partitions; each yields (m, l, acc) and the partials are merged with the
+    log-sum-exp rule. Partitions with no visible key carry m=-inf, l=0.
+
+    Returns (out ``[Hq, D]``, lse ``[Hq]``)."""
+    q = np.asarray(q, dtype=dtype)
+    hq, d = q.shape
+    kk = _expand_kv(np.asarray(k[:kv_len], dtype=dtype), hq)
+    vv = _expand_kv(np.asarray(v[:kv_len], dtype=dtype), hq)
+    p = kv_len - 1
+    vis = visibility(np.array([p]), kv_len, window)[0]
+    per = -(-kv_len // num_splits)
+    ms = np.full((num_splits, hq), -np.inf, dtype=dtype)
+    ls = np.zeros((num_splits, hq), dtype=dtype)
+    accs = np.zeros((num_splits, hq, d), dtype=dtype)
+    for sidx in range(num_splits):
+        lo, hi = sidx * per, min(kv_len, (sidx + 1) * per)
+        if lo >= hi:
+            continue
+        s = np.einsum("hd,lhd->hl", q * dtype(scale), kk[lo:hi])
+        if softcap and softcap > 0.0:
+            s = dtype(softcap) * np.tanh(s / dtype(softcap))
+        s = np.where(vis[None, lo:hi], s, -np.inf)
+        m = s.max(axis=-1)
+        if not np.isfinite(m).any():
+            continue
+        msafe = np.where(np.isfinite(m), m, 0.0)
+        e = np.exp(s - msafe[:, None])
+        ms[sidx] = m
+        ls[sidx] = e.sum(axis=-1)
+        accs[sidx] = np.einsum("hl,lhd->hd", e, vv[lo:hi])
+    mg = ms.max(axis=0)
+    mg_safe = np.where(np.isfinite(mg), mg, 0.0)
+    w = np.where(np.isfinite(ms), np.exp(ms - mg_safe[None, :]), 0.0)
+    l = (w * ls).sum(axis=0)
+    acc = (w[:, :, None] * accs).sum(axis=0)
+    out = np.divide(acc, l[:, None], out=np.zeros_like(acc), where=l[:, None] > 0)
+    lse = mg + np.log(np.where(l > 0, l, 1.0))
+    return out, lse
+
+
+# --------------------------------------------------------------------------
+# int8 per-(kv head, channel) KV cache
+# --------------------------------------------------------------------------
+def quantize_kv_int8(x: np.ndarray):
+    """x ``[L, Hkv, D]`` fp32 -> (int8 ``[L,Hkv,D]``, scale fp32 ``[Hkv,D]``) with
+    scale = absmax/127 per (head, channel), value = clamp(round(x/scale), +-127)."""
+    x = np.asarray(x, dtype=np.float32)
+    absmax = np.abs(x).max(axis=0)
+    scale = (absmax / np.float32(127.0)).astype(np.float32)
+    safe = np.where(scale > 0, scale, np.float32(1.0))
+    qv = np.clip(np.rint(x / safe[None]), -127, 127).astype(np.int8)
+    return qv, scale
+
+
+def dequantize_kv_int8(qv: np.ndarray, scale: np.ndarray) -> np.ndarray:
+    return qv.astype(np.float32) * np.asarray(scale, dtype=np.float32)[None]
+
+
+# --------------------------------------------------------------------------
+# Prefill chunk planner (reference: utils.cc:300-330)
+# --------------------------------------------------------------------------
+def prefill_work_groups(runner_lengths, input_length: int):
+    """``runner_lengths``: the static sequence lengths of the available prefill
+    runners. Returns ``[(runner_length, tokens_in_this_call), ...]``: the longest
+    runner while a full one fits, then one call on the shortest runner that still
+    holds the remainder."""
+    lens = sorted(set(int(x) for x in runner_lengths), reverse=True)
+    if not lens:
+        raise ValueError("no prefill runner")
+    out = []
+    longest = lens[0]
+    while input_length >= longest:
+        out.append((longest, longest))
+        input_length -= longest
+    if input_length > 0:
+        pick = lens[0]
+        for cand in lens:
+            if cand >= input_length:
+                pick = cand
+        out.append((pick, input_length))
+    return out
+
+
+# --------------------------------------------------------------------------
+# Executor state machine (reference: executor.cc:157-276, 416-534, 568-574)
+# --------------------------------------------------------------------------
+class OracleExecutor:
+    """Bookkeeping twin of the reference executor. ``run(kind, tokens, positions)``
+    is invoked where the reference calls ``compiled_model_.Run``; it records the
+    (token, position) pairs each call executes.
+
+    ``execute_single_pending`` selects between the reference behaviour for a
+    1-id prefill chunk (False: the loop at executor.cc:187 does not run, so a
+    pending token is overwritten and never executed) and the corrected behaviour
+    of the HIP executor (True: the pending token is executed first).
+    """
+
+    def __init__(self, runner_lengths=(1024,), max_num_tokens: int = 4096,
+                 execute_single_pending: bool = True):
+        self.runner_lengths = tuple(runner_lengths)
+        self.max_num_tokens = max_num_tokens
+        self.execute_single_pending = execute_single_pending
+        self.current_step = 0
+        self.next_input_token_id = -1
+        self.calls = []
+
+    def get_current_step(self) -> int:
+        return self.current_step + (1 if self.next_input_token_id != -1 else 0)
+
+    def reset(self):
+        self.current_step = 0
+        self.next_input_token_id = -1
+
+    def prefill(self, ids):
+        ids = [int(x) for x in ids]
+        if not ids:
+            raise ValueError("Prefill token ids must be non-empty.")
+        for _, n in prefill_work_groups(self.runner_lengths, len(ids)):
+            self._prefill_chunk(ids[:n])
+            ids = ids[n:]
+        assert not ids
+
+    def _prefill_chunk(self, ids):
+        toks, pos = [], []
+        i = 0
+        limit = len(ids) - 1
+        if self.execute_single_pending and limit == 0 and self.next_input_token_id != -1:
+            toks.append(self.next_input_token_id)
+            pos.append(self.current_step)
+            self.next_input_token_id = -1
+            self.current_step += 1
+        while i < limit:
+            if self.next_input_token_id != -1:
+                toks.append(self.next_input_token_id)
+                self.next_input_token_id = -1
+            else:
+                toks.append(ids[i])
+                i += 1
+            pos.append(self.current_step)
+            self.current_step += 1
+        self.next_input_token_id = ids[-1]
+        self.calls.append(("prefill", toks, pos))
+
+    def decode(self, explicit_id=None) -> int:
+        tok = self.next_input_token_id if explicit_id is None else int(explicit_id)
+        if tok == -1:
+            raise ValueError("No id available to be decoded.")
+        self.next_input_token_id = -1
+        self.calls.append(("decode", [tok], [self.current_step]))
+        self.current_step += 1
+        return tok
+
+
+# --------------------------------------------------------------------------
+# Synthetic inputs of the five benchmark configurations
+# --------------------------------------------------------------------------
+SEED_BASE = 0xC0FFEE
+
+
+def config_rng(idx: int) -> np.random.Generator:
+    return np.random.default_rng(SEED_BASE + idx)
+
+
+def c2_layer_window(layer: int, window: int = 512) -> int:
+    """5:1 local:global pattern: layer is global iff (layer + 1) % 6 == 0."""
+    return 0 if (layer + 1) % 6 == 0 else window
+
+
+def rel_err(a, b) -> float:
+    """Norm-wise relative error max|a-b| / max|b| per output tensor."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    den = np.abs(b).max()
+    return float(np.abs(a - b).max() / (den if den > 0 else 1.0))
