@@ -1,0 +1,199 @@
+/*
+ * mi355_attn.h - C ABI of the MI355X (gfx950) attention library.
+ *
+ * The library owns a KV cache in HBM and runs scaled-dot-product attention over
+ * it: causal prefill (global and sliding-window layers) and one-token decode
+ * (GQA/MQA, split-KV partitions merged by log-sum-exp). It is the thin layer a
+ * C++ LlmExecutor implementation calls where the reference executor calls
+ * litert::CompiledModel::Run.
+ *
+ * Conventions follow the reference's own dlopen'd plugin ABI
+ * (runtime/components/sampler_factory.cc:34-57,119-133,156-188):
+ *   - every call returns an absl::StatusCode integer (0 = OK);
+ *   - `char** error_msg` (may be NULL) receives a malloc'd message that the
+ *     caller releases with free();
+ *   - plain C types only; nothing throws across the boundary.
+ * A handle is not thread-safe: like the reference executor it is driven from
+ * one worker thread (runtime/core/engine_impl.cc:185-186).
+ *
+ * Tensor layouts at the boundary (row-major, dense):
+ *   q, out : [n][num_q_heads][head_dim]          io_dtype
+ *   k, v   : [n][num_kv_heads][head_dim]         kv_dtype
+ *   scales : [num_kv_heads][head_dim]            float32 (int8 cache only)
+ * Query head h reads KV head h / (num_q_heads / num_kv_heads).
+ * Key j is visible to the query at absolute position p iff j <= p and, on a
+ * layer with window W > 0, p - j < W.
+ */
+#ifndef MI355_ATTN_H_
+#define MI355_ATTN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mi355_attn mi355_attn;
+
+/* Element types. */
+enum {
+  MI355_ATTN_F32 = 0,
+  MI355_ATTN_F16 = 1,
+  MI355_ATTN_BF16 = 2,
+  MI355_ATTN_I8 = 3 /* kv_dtype only: symmetric int8, per-(kv head, channel) scale */
+};
+
+/* absl::StatusCode values used by this library. */
+enum {
+  MI355_ATTN_OK = 0,
+  MI355_ATTN_INVALID_ARGUMENT = 3,
+  MI355_ATTN_RESOURCE_EXHAUSTED = 8,
+  MI355_ATTN_FAILED_PRECONDITION = 9,
+  MI355_ATTN_OUT_OF_RANGE = 11,
+  MI355_ATTN_UNIMPLEMENTED = 12,
+  MI355_ATTN_INTERNAL = 13,
+  MI355_ATTN_UNAVAILABLE = 14
+};
+
+/*
+ * Static description of one executor's attention stack. Plays the part that the
+ * .tflite signature shapes plus LlmExecutorSettings play in the reference
+ * (runtime/executor/llm_executor_settings.h:95-154: max_num_tokens is the KV
+ * capacity; runtime/executor/llm_litert_compiled_model_executor.cc:716-761:
+ * one K and one V tensor per layer).
+ */
+typedef struct mi355_attn_config {
+  uint32_t struct_size;        /* sizeof(mi355_attn_config) */
+  int32_t num_layers;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;            /* 256 */
+  int32_t max_tokens;          /* KV rows per sequence */
+  int32_t max_seqs;            /* sequences (cache slots) held at once */
+  int32_t kv_dtype;            /* MI355_ATTN_* */
+  int32_t io_dtype;            /* MI355_ATTN_F32 / F16 / BF16 */
+  float scale;                 /* 0 => head_dim^-0.5 */
+  float softcap;               /* 0 => off; else cap * tanh(s / cap) */
+  const int32_t* layer_window; /* [num_layers], 0 = global layer; NULL = all global */
+  int32_t device;              /* HIP device ordinal */
+  int32_t host_io;             /* 0: q/k/v/out/scales are device pointers;
+                                  1: host pointers, staged by the library and
+                                     every call returns with results in place */
+  int32_t own_stream;          /* 1: run on a new non-blocking stream owned by the handle
+                                  (`stream` is ignored); 0: run on `stream` */
+  void* stream;                /* hipStream_t; NULL = the HIP default stream */
+} mi355_attn_config;
+
+/*
+ * Builds the handle and its zero-initialised KV cache.
+ * Replaces: LlmLiteRtCompiledModelExecutor::Create's KV-buffer allocation
+ * (runtime/executor/llm_litert_compiled_model_executor.cc:705-761).
+ * kUnavailable when no gfx950 device can be used.
+ */
+int mi355_attn_create(const mi355_attn_config* config, mi355_attn** out, char** error_msg);
+
+void mi355_attn_destroy(mi355_attn* handle);
+
+/*
+ * Writes n new K/V rows of one layer of sequence `seq` at rows pos .. pos+n-1.
+ * Replaces: the in-graph KV update behind compiled_model_.Run, visible in tree
+ * as the cache tensors being both inputs and outputs of every signature
+ * (llm_litert_compiled_model_executor.cc:733-757) and as the explicit
+ * cache-update signature of the NPU flow
+ * (llm_litert_npu_compiled_model_executor.cc:105-110,1294-1333).
+ * For an int8 cache k and v hold int8 values; set the scales with
+ * mi355_attn_kv_set_scales.
+ */
+int mi355_attn_kv_append(mi355_attn* handle, int32_t layer, int32_t seq, int32_t pos, int32_t n,
+                         const void* k, const void* v, char** error_msg);
+
+/* int8 cache: per-(kv head, channel) dequantisation scales of (layer, seq). */
+int mi355_attn_kv_set_scales(mi355_attn* handle, int32_t layer, int32_t seq, const float* k_scale,
+                             const float* v_scale, char** error_msg);
+
+/* Reads cache rows pos .. pos+n-1 back in boundary layout (tests, debugging). */
+int mi355_attn_kv_read(mi355_attn* handle, int32_t layer, int32_t seq, int32_t pos, int32_t n, void* k_out,
+                       void* v_out, char** error_msg);
+
+/*
+ * Prefill attention of one layer: n query rows at absolute positions
+ * q_pos0 .. q_pos0+n-1 of sequence `seq` over cache rows [0, q_pos0+n), causal,
+ * windowed on local layers. The rows' own K/V must already be appended.
+ * Replaces: the attention inside compiled_model_.Run(prefill_signature, ...)
+ * (llm_litert_compiled_model_executor.cc:271) together with the causal mask
+ * the executor builds for it
+ * (runtime/executor/litert_compiled_model_executor_utils.cc:332-397).
+ */
+int mi355_attn_prefill(mi355_attn* handle, int32_t layer, int32_t seq, int32_t q_pos0, int32_t n,
+                       const void* q, void* out, char** error_msg);
+
+/*
+ * Same for n_layers consecutive layers in one launch; q and out are
+ * [n_layers][n][num_q_heads][head_dim]. The layers' problems are independent
+ * (throughput sweeps; a real forward pass calls mi355_attn_prefill per layer).
+ */
+int mi355_attn_prefill_layers(mi355_attn* handle, int32_t layer_begin, int32_t n_layers, int32_t seq,
+                              int32_t q_pos0, int32_t n, const void* q, void* out, char** error_msg);
+
+/*
+ * One-token decode attention of one layer for `batch` sequences.
+ * seq_ids[b] (host array, NULL = 0..batch-1) names the cache slot and
+ * kv_lens[b] (host array) the number of valid rows, the new token's row
+ * included: the query of item b sits at position kv_lens[b]-1.
+ * num_splits >= 1 cuts each key range into that many partitions whose partial
+ * (max, sum, accumulator) are merged by log-sum-exp; 0 lets the library choose.
+ * Replaces: the attention inside compiled_model_.Run("decode", ...)
+ * (llm_litert_compiled_model_executor.cc:407,522) and its one-row mask
+ * (:485-492).
+ */
+int mi355_attn_decode(mi355_attn* handle, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,
+                      int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg);
+
+/* n_layers consecutive layers in one launch; q, out [n_layers][batch][Hq][D]. */
+int mi355_attn_decode_layers(mi355_attn* handle, int32_t layer_begin, int32_t n_layers,
+                             const int32_t* seq_ids, const int32_t* kv_lens, int32_t batch, const void* q,
+                             void* out, int32_t num_splits, char** error_msg);
+
+/*
+ * Forgets the rows of sequence `seq` (seq < 0: all). Like
+ * LlmLiteRtCompiledModelExecutor::Reset
+ * (llm_litert_compiled_model_executor.cc:568-574) the cache memory itself is
+ * not cleared; stale rows are never visible because visibility is bounded by
+ * the positions the caller passes.
+ */
+int mi355_attn_reset(mi355_attn* handle, int32_t seq, char** error_msg);
+
+/* Blocks until all work queued on the handle's stream has finished. */
+int mi355_attn_sync(mi355_attn* handle, char** error_msg);
+
+/* The stream work is queued on (hipStream_t). */
+void* mi355_attn_stream(mi355_attn* handle);
+
+/*
+ * Duration in milliseconds of the attention kernel of the most recent
+ * prefill/decode call, measured with HIP events on the handle's stream
+ * (the split-merge pass is excluded). Blocks until that call has finished.
+ * Timing is recorded only after mi355_attn_set_timing(handle, 1).
+ */
+int mi355_attn_set_timing(mi355_attn* handle, int32_t enabled);
+float mi355_attn_last_kernel_ms(mi355_attn* handle);
+
+/*
+ * Tuning and cross-check switches (return kInvalidArgument for unknown names):
+ *   "decode_waves"     2 or 4 waves per decode workgroup (default 4)
+ *   "decode_pipeline"  0/1 keep the next block's loads in flight (default 1)
+ *   "rowwise_prefill"  0/1 run prefill row by row through the decode kernel
+ *                      (the only path for fp32 and int8 caches)
+ */
+int mi355_attn_set_option(mi355_attn* handle, const char* name, int32_t value);
+
+/* Bytes of HBM held by the KV cache of this handle. */
+uint64_t mi355_attn_cache_bytes(const mi355_attn* handle);
+
+/* Library version string, e.g. "mi355_attn 0.1 (gfx950)". */
+const char* mi355_attn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_ATTN_H_ */

@@ -1,0 +1,136 @@
+// Shared between the host side of the C ABI and the gfx950 kernels: element
+// types, the KV-cache layout in HBM and the kernel argument blocks.
+//
+// KV-cache layout (one "plane" per layer x sequence x KV head x {K,V}).
+// A plane holds `cap` token rows (cap = max_tokens rounded up to 64) of
+// head_dim elements, stored so that every MFMA operand a wave needs is one
+// 16-byte load per lane and every wave-wide load instruction covers 1 KiB of
+// consecutive bytes:
+//
+//   EPC = 16 / sizeof(element)  elements per 16-byte chunk (4 f32, 8 f16/bf16, 16 i8)
+//
+//   K plane: tiles of 16 tokens. Inside a tile, chunk c = d / EPC of token
+//   r = t % 16 sits at byte (c * 16 + r) * 16. A lane (r = lane % 16,
+//   g = lane / 16) loading chunk 4*j + g of token r for j = 0,1,.. holds the
+//   A operand (16 tokens x K-slice) of S^T = K . Q^T directly.
+//
+//   V plane: blocks of VB = 4 * EPC tokens. Token tb = t % VB of a block is
+//   tile T = tb / 16, group g = (tb % 16) / 4, slot = 4 * T + tb % 4; element
+//   (t, d) sits at byte ((d / 16 * 4 + g) * 16 + d % 16) * 16 + slot * sizeof.
+//   The 16 bytes of lane (r = d % 16, g) are the A operand (16 channels x
+//   token-slice) of O^T = V^T . P^T, and their token order matches the
+//   accumulator layout in which S^T leaves the first MFMA, so P never moves
+//   between lanes.
+#ifndef LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_
+#define LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define MI355_HD __host__ __device__ inline
+#else
+#define MI355_HD inline
+#endif
+
+namespace mi355 {
+
+enum DType : int32_t { kF32 = 0, kF16 = 1, kBF16 = 2, kI8 = 3 };
+
+MI355_HD int dtype_size(int dt) { return dt == kF32 ? 4 : (dt == kI8 ? 1 : 2); }
+
+constexpr int kTokenAlign = 64;  // planes hold a multiple of 64 rows
+constexpr int kMaxGroup = 16;    // query heads per KV head handled by one MFMA column block
+
+MI355_HD int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+struct CacheGeom {
+  int32_t num_layers, max_seqs, hkv, head_dim, cap, esize;
+  int64_t plane_bytes;  // cap * head_dim * esize
+  // plane index order: [layer][seq][kv_head][K=0 / V=1]
+  MI355_HD int64_t plane_offset(int layer, int seq, int kvh, int is_v) const {
+    return ((((int64_t)layer * max_seqs + seq) * hkv + kvh) * 2 + is_v) * plane_bytes;
+  }
+  // scales: float [layer][seq][K=0 / V=1][kv_head][head_dim]
+  MI355_HD int64_t scale_offset(int layer, int seq, int is_v, int kvh) const {
+    return ((((int64_t)layer * max_seqs + seq) * 2 + is_v) * hkv + kvh) * head_dim;
+  }
+};
+
+// Byte offset of the 16-byte chunk holding elements [c*EPC, (c+1)*EPC) of token t in a K plane.
+MI355_HD int64_t k_chunk_offset(int t, int c, int head_dim, int esize) {
+  const int64_t tile_bytes = (int64_t)16 * head_dim * esize;
+  return (int64_t)(t >> 4) * tile_bytes + ((int64_t)c * 16 + (t & 15)) * 16;
+}
+
+// Byte offset of element (t, d) in a V plane.
+MI355_HD int64_t v_elem_offset(int t, int d, int head_dim, int esize) {
+  const int epc = 16 / esize;
+  const int vb = 4 * epc;
+  const int64_t block_bytes = (int64_t)vb * head_dim * esize;
+  const int tb = t % vb;
+  const int T = tb >> 4, g = (tb & 15) >> 2, slot = 4 * T + (tb & 3);
+  return (int64_t)(t / vb) * block_bytes + ((int64_t)((d >> 4) * 4 + g) * 16 + (d & 15)) * 16 +
+         (int64_t)slot * esize;
+}
+
+// Arguments of the decode kernels (passed by value).
+struct DecodeArgs {
+  const void* q;             // [n_layers][batch][hq][D] io dtype
+  void* out;                 // same shape
+  const uint8_t* cache;      // base of all planes
+  const float* scales;       // int8 cache only
+  float* ws_acc;             // [items][hq][num_splits][D] partial accumulators
+  float* ws_ml;              // [items][hq][num_splits][2] partial (max, sum)
+  const int32_t* kv_lens;    // [batch]
+  const int32_t* seq_ids;    // [batch] or nullptr
+  const int32_t* layer_window;  // [num_layers]
+  CacheGeom geom;
+  int32_t hq, group;
+  int32_t layer_begin, n_layers, batch;
+  int32_t num_splits;
+  int32_t max_kv_len;        // max over kv_lens (host computed), sizes the partitions
+  float scale;               // softmax scale
+  float softcap;
+};
+
+// Tokens per split-KV partition for a layer with the given window: the same
+// formula runs in the attention kernel and in the merge kernel.
+MI355_HD int decode_partition_tokens(int max_kv_len, int window, int num_splits) {
+  int span = max_kv_len;
+  if (window > 0 && window + (kTokenAlign - 1) < span) span = window + (kTokenAlign - 1);
+  int per = (span + num_splits - 1) / num_splits;
+  per = (per + kTokenAlign - 1) / kTokenAlign * kTokenAlign;
+  return per < kTokenAlign ? kTokenAlign : per;
+}
+
+// First visible key and the 64-aligned row at which partition 0 starts.
+MI355_HD void decode_visible_range(int kv_len, int window, int* vlo, int* start) {
+  int lo = 0;
+  if (window > 0 && kv_len > window) lo = kv_len - window;
+  *vlo = lo;
+  *start = lo & ~(kTokenAlign - 1);
+}
+
+struct PrefillArgs {
+  const void* q;   // [n_layers][n][hq][D]
+  void* out;
+  const uint8_t* cache;
+  const float* scales;
+  const int32_t* layer_window;
+  CacheGeom geom;
+  int32_t hq, group;
+  int32_t layer_begin, n_layers;
+  int32_t seq, q_pos0, n;
+  float scale, softcap;
+};
+
+struct KvCopyArgs {
+  uint8_t* cache;
+  CacheGeom geom;
+  int32_t layer, seq, pos, n;
+  void* k;  // [n][hkv][D] boundary layout (source for append, destination for read)
+  void* v;
+};
+
+}  // namespace mi355
+#endif  // LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_

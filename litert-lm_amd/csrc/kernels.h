@@ -1,0 +1,34 @@
+// Launchers of the gfx950 kernels; the C ABI in mi355_attn.hip validates
+// shapes on the host and then calls these.
+#ifndef LITERT_LM_AMD_CSRC_KERNELS_H_
+#define LITERT_LM_AMD_CSRC_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+
+#include "attn_params.h"
+
+namespace mi355 {
+
+struct DecodeTuning {
+  int waves = 4;         // waves per workgroup (2 or 4)
+  bool pipeline = true;  // keep the next block's loads in flight during arithmetic
+};
+
+bool decode_supported(int kv_dtype, int io_dtype, int head_dim);
+
+// Queues the decode attention kernel (bracketed by ev0/ev1 when non-null) and,
+// for num_splits > 1, the log-sum-exp merge kernel.
+hipError_t launch_decode(const DecodeArgs& args, int kv_dtype, int io_dtype, const DecodeTuning& tuning,
+                         hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1);
+
+bool prefill_supported(int kv_dtype, int io_dtype, int head_dim);
+
+hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, hipStream_t stream,
+                          hipEvent_t ev0, hipEvent_t ev1);
+
+// Scatter n boundary-layout rows into the cache planes / gather them back.
+hipError_t launch_kv_append(const KvCopyArgs& args, hipStream_t stream);
+hipError_t launch_kv_read(const KvCopyArgs& args, hipStream_t stream);
+
+}  // namespace mi355
+#endif  // LITERT_LM_AMD_CSRC_KERNELS_H_

@@ -1,0 +1,79 @@
+// KV-cache update and read-back kernels: move token rows between the boundary
+// layout [n][kv_heads][head_dim] and the MFMA-operand layout of the planes.
+//
+// Replaces the in-graph cache update that the reference reaches through
+// compiled_model_.Run (cache tensors are inputs and outputs of every
+// signature, runtime/executor/llm_litert_compiled_model_executor.cc:733-757).
+#include <hip/hip_runtime.h>
+
+#include "attn_params.h"
+#include "kernels.h"
+#include "mfma_util.h"
+
+namespace mi355 {
+namespace {
+
+// One thread per 16-byte chunk of a source row. ESZ = element bytes.
+template <int ESZ, bool APPEND>
+__global__ void __launch_bounds__(256) kv_copy_kernel(const KvCopyArgs a) {
+  constexpr int EPC = 16 / ESZ;
+  const int D = a.geom.head_dim;
+  const int chunks = D / EPC;
+  const int64_t total = (int64_t)a.n * a.geom.hkv * chunks;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  // token index fastest: consecutive threads touch consecutive 16-byte chunks of a K tile
+  const int i = (int)(idx % a.n);
+  const int c = (int)((idx / a.n) % chunks);
+  const int h = (int)(idx / ((int64_t)a.n * chunks));
+  const int t = a.pos + i;
+  uint8_t* kplane = a.cache + a.geom.plane_offset(a.layer, a.seq, h, 0);
+  uint8_t* vplane = kplane + a.geom.plane_bytes;
+  const int64_t row = ((int64_t)i * a.geom.hkv + h) * D + (int64_t)c * EPC;  // element index in k / v
+  uint8_t* kb = reinterpret_cast<uint8_t*>(a.k) + row * ESZ;
+  uint8_t* vb = reinterpret_cast<uint8_t*>(a.v) + row * ESZ;
+  u4* kc = reinterpret_cast<u4*>(kplane + k_chunk_offset(t, c, D, ESZ));
+  if constexpr (APPEND) {
+    *kc = *reinterpret_cast<const u4*>(kb);
+    const u4 vw = *reinterpret_cast<const u4*>(vb);
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(&vw);
+#pragma unroll
+    for (int e = 0; e < EPC; ++e) {
+      uint8_t* dst = vplane + v_elem_offset(t, c * EPC + e, D, ESZ);
+      if constexpr (ESZ == 4) *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src + 4 * e);
+      else if constexpr (ESZ == 2) *reinterpret_cast<uint16_t*>(dst) = *reinterpret_cast<const uint16_t*>(src + 2 * e);
+      else *dst = src[e];
+    }
+  } else {
+    *reinterpret_cast<u4*>(kb) = *kc;
+    u4 vw;
+    uint8_t* dstb = reinterpret_cast<uint8_t*>(&vw);
+#pragma unroll
+    for (int e = 0; e < EPC; ++e) {
+      const uint8_t* s = vplane + v_elem_offset(t, c * EPC + e, D, ESZ);
+      if constexpr (ESZ == 4) *reinterpret_cast<uint32_t*>(dstb + 4 * e) = *reinterpret_cast<const uint32_t*>(s);
+      else if constexpr (ESZ == 2) *reinterpret_cast<uint16_t*>(dstb + 2 * e) = *reinterpret_cast<const uint16_t*>(s);
+      else dstb[e] = *s;
+    }
+    *reinterpret_cast<u4*>(vb) = vw;
+  }
+}
+
+template <bool APPEND>
+hipError_t launch_copy(const KvCopyArgs& a, hipStream_t stream) {
+  if (a.n <= 0) return hipSuccess;
+  const int esz = a.geom.esize;
+  const int64_t total = (int64_t)a.n * a.geom.hkv * (a.geom.head_dim / (16 / esz));
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (esz == 4) hipLaunchKernelGGL((kv_copy_kernel<4, APPEND>), grid, dim3(256), 0, stream, a);
+  else if (esz == 2) hipLaunchKernelGGL((kv_copy_kernel<2, APPEND>), grid, dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((kv_copy_kernel<1, APPEND>), grid, dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_kv_append(const KvCopyArgs& a, hipStream_t stream) { return launch_copy<true>(a, stream); }
+hipError_t launch_kv_read(const KvCopyArgs& a, hipStream_t stream) { return launch_copy<false>(a, stream); }
+
+}  // namespace mi355

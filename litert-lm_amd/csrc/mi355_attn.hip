@@ -1,0 +1,625 @@
+// C ABI of the MI355X attention library (see include/mi355_attn.h): handle
+// lifetime, host-side validation of every shape before a kernel is launched,
+// status/error-message conventions, staging for host-pointer callers.
+#include "../../include/mi355_attn.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "attn_params.h"
+#include "kernels.h"
+
+using namespace mi355;
+
+namespace {
+
+constexpr int kRingSlots = 64;
+constexpr int kMaxSplits = 256;
+
+int fail(char** error_msg, int code, const char* fmt, ...) {
+  if (error_msg) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    const size_t len = strlen(buf) + 1;
+    char* msg = static_cast<char*>(malloc(len));
+    if (msg) memcpy(msg, buf, len);
+    *error_msg = msg;
+  }
+  return code;
+}
+
+#define HIP_OR_RETURN(expr)                                                                       \
+  do {                                                                                            \
+    hipError_t e_ = (expr);                                                                       \
+    if (e_ != hipSuccess)                                                                         \
+      return fail(error_msg, e_ == hipErrorOutOfMemory ? MI355_ATTN_RESOURCE_EXHAUSTED            \
+                                                       : MI355_ATTN_INTERNAL,                     \
+                  "%s failed: %s", #expr, hipGetErrorString(e_));                                 \
+  } while (0)
+
+__global__ void iota_items_kernel(int32_t* lens, int32_t* seq_ids, int n, int q_pos0, int seq) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    lens[i] = q_pos0 + i + 1;
+    seq_ids[i] = seq;
+  }
+}
+
+}  // namespace
+
+struct mi355_attn {
+  mi355_attn_config cfg{};
+  CacheGeom geom{};
+  int device = 0;
+  hipStream_t stream = nullptr;
+  bool own_stream = false;
+  uint8_t* cache = nullptr;
+  uint64_t cache_bytes = 0;
+  float* scales = nullptr;
+  int32_t* d_window = nullptr;
+  std::vector<int32_t> window;
+  std::vector<int32_t> filled;  // [layer][seq] rows written since the last reset
+  // split-KV workspace
+  float* ws_acc = nullptr;
+  float* ws_ml = nullptr;
+  size_t ws_slots = 0;
+  // ring of (kv_lens, seq_ids) uploads
+  int32_t* h_ring = nullptr;
+  int32_t* d_ring = nullptr;
+  hipEvent_t ring_ev[kRingSlots] = {};
+  bool ring_used[kRingSlots] = {};
+  int ring_next = 0;
+  int ring_slot_ints = 0;
+  // per-row items of the row-wise prefill path
+  int32_t* d_items = nullptr;
+  size_t d_items_cap = 0;
+  // staging for host_io
+  void* stage[4] = {nullptr, nullptr, nullptr, nullptr};
+  size_t stage_cap[4] = {0, 0, 0, 0};
+  // timing
+  bool timing = false;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  bool timed = false;
+  DecodeTuning tuning;
+  bool rowwise_prefill = false;  // force the row-wise prefill path (cross-checks)
+};
+
+namespace {
+
+int io_size(const mi355_attn* h) { return dtype_size(h->cfg.io_dtype); }
+int kv_size(const mi355_attn* h) { return dtype_size(h->cfg.kv_dtype); }
+
+int ensure_stage(mi355_attn* h, int which, size_t bytes, char** error_msg) {
+  if (h->stage_cap[which] >= bytes) return 0;
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  if (h->stage[which]) HIP_OR_RETURN(hipFree(h->stage[which]));
+  h->stage[which] = nullptr;
+  h->stage_cap[which] = 0;
+  const size_t cap = std::max(bytes, (size_t)1 << 20);
+  HIP_OR_RETURN(hipMalloc(&h->stage[which], cap));
+  h->stage_cap[which] = cap;
+  return 0;
+}
+
+// Device view of a caller buffer that the kernels read.
+int stage_in(mi355_attn* h, int which, const void* p, size_t bytes, const void** dev, char** error_msg) {
+  if (!h->cfg.host_io) {
+    *dev = p;
+    return 0;
+  }
+  if (int rc = ensure_stage(h, which, bytes, error_msg)) return rc;
+  HIP_OR_RETURN(hipMemcpyAsync(h->stage[which], p, bytes, hipMemcpyHostToDevice, h->stream));
+  *dev = h->stage[which];
+  return 0;
+}
+
+int stage_out_begin(mi355_attn* h, int which, void* p, size_t bytes, void** dev, char** error_msg) {
+  if (!h->cfg.host_io) {
+    *dev = p;
+    return 0;
+  }
+  if (int rc = ensure_stage(h, which, bytes, error_msg)) return rc;
+  *dev = h->stage[which];
+  return 0;
+}
+
+int stage_out_end(mi355_attn* h, int which, void* p, size_t bytes, char** error_msg) {
+  if (!h->cfg.host_io) return 0;
+  HIP_OR_RETURN(hipMemcpyAsync(p, h->stage[which], bytes, hipMemcpyDeviceToHost, h->stream));
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  return 0;
+}
+
+int ensure_workspace(mi355_attn* h, size_t slots, char** error_msg) {
+  if (h->ws_slots >= slots) return 0;
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  if (h->ws_acc) HIP_OR_RETURN(hipFree(h->ws_acc));
+  if (h->ws_ml) HIP_OR_RETURN(hipFree(h->ws_ml));
+  h->ws_acc = h->ws_ml = nullptr;
+  h->ws_slots = 0;
+  HIP_OR_RETURN(hipMalloc(&h->ws_acc, slots * h->cfg.head_dim * sizeof(float)));
+  HIP_OR_RETURN(hipMalloc(&h->ws_ml, slots * 2 * sizeof(float)));
+  h->ws_slots = slots;
+  return 0;
+}
+
+// Uploads kv_lens (and seq_ids) through a ring of pinned slots so that calls
+// can be queued back to back without waiting for earlier uploads.
+int upload_items(mi355_attn* h, const int32_t* seq_ids, const int32_t* kv_lens, int batch,
+                 const int32_t** d_lens, const int32_t** d_seq, char** error_msg) {
+  const int slot = h->ring_next;
+  h->ring_next = (slot + 1) % kRingSlots;
+  if (h->ring_used[slot]) HIP_OR_RETURN(hipEventSynchronize(h->ring_ev[slot]));
+  int32_t* hs = h->h_ring + (size_t)slot * h->ring_slot_ints;
+  int32_t* ds = h->d_ring + (size_t)slot * h->ring_slot_ints;
+  memcpy(hs, kv_lens, sizeof(int32_t) * batch);
+  if (seq_ids) memcpy(hs + batch, seq_ids, sizeof(int32_t) * batch);
+  const size_t bytes = sizeof(int32_t) * batch * (seq_ids ? 2 : 1);
+  HIP_OR_RETURN(hipMemcpyAsync(ds, hs, bytes, hipMemcpyHostToDevice, h->stream));
+  HIP_OR_RETURN(hipEventRecord(h->ring_ev[slot], h->stream));
+  h->ring_used[slot] = true;
+  *d_lens = ds;
+  *d_seq = seq_ids ? ds + batch : nullptr;
+  return 0;
+}
+
+int check_layers(const mi355_attn* h, int layer_begin, int n_layers, char** error_msg) {
+  if (layer_begin < 0 || n_layers < 1 || layer_begin + n_layers > h->cfg.num_layers)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "layers [%d, %d) outside [0, %d)", layer_begin,
+                layer_begin + n_layers, h->cfg.num_layers);
+  return 0;
+}
+
+void fill_decode_common(const mi355_attn* h, DecodeArgs* a) {
+  a->cache = h->cache;
+  a->scales = h->scales;
+  a->ws_acc = h->ws_acc;
+  a->ws_ml = h->ws_ml;
+  a->layer_window = h->d_window;
+  a->geom = h->geom;
+  a->hq = h->cfg.num_q_heads;
+  a->group = h->cfg.num_q_heads / h->cfg.num_kv_heads;
+  a->scale = h->cfg.scale;
+  a->softcap = h->cfg.softcap;
+}
+
+int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq_ids, const int32_t* kv_lens,
+                int batch, const void* q, void* out, int num_splits, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (int rc = check_layers(h, layer_begin, n_layers, error_msg)) return rc;
+  if (!kv_lens || !q || !out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null kv_lens, q or out");
+  if (batch < 1 || batch > h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "batch %d outside [1, max_seqs=%d]", batch,
+                h->cfg.max_seqs);
+  if (num_splits < 0 || num_splits > kMaxSplits)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "num_splits %d outside [0, %d]", num_splits, kMaxSplits);
+  if (!decode_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim))
+    return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "decode: unsupported kv/io dtype pair %d/%d",
+                h->cfg.kv_dtype, h->cfg.io_dtype);
+  int max_len = 0;
+  for (int b = 0; b < batch; ++b) {
+    const int seq = seq_ids ? seq_ids[b] : b;
+    if (seq < 0 || seq >= h->cfg.max_seqs)
+      return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq_ids[%d]=%d outside [0, %d)", b, seq,
+                  h->cfg.max_seqs);
+    const int len = kv_lens[b];
+    if (len < 1 || len > h->cfg.max_tokens)
+      return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "kv_lens[%d]=%d outside [1, max_tokens=%d]", b, len,
+                  h->cfg.max_tokens);
+    for (int l = layer_begin; l < layer_begin + n_layers; ++l)
+      if (len > h->filled[(size_t)l * h->cfg.max_seqs + seq])
+        return fail(error_msg, MI355_ATTN_OUT_OF_RANGE,
+                    "kv_lens[%d]=%d but only %d rows of layer %d, sequence %d were appended", b, len,
+                    h->filled[(size_t)l * h->cfg.max_seqs + seq], l, seq);
+    max_len = std::max(max_len, len);
+  }
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const int items = n_layers * batch;
+  if (num_splits == 0) {
+    // enough workgroups to cover the chip a few times, partitions of >= 128 tokens
+    const int want = (2048 + items * h->cfg.num_kv_heads - 1) / (items * h->cfg.num_kv_heads);
+    num_splits = std::max(1, std::min({want, (max_len + 127) / 128, 64}));
+  }
+  DecodeArgs a{};
+  if (num_splits > 1)
+    if (int rc = ensure_workspace(h, (size_t)items * h->cfg.num_q_heads * num_splits, error_msg)) return rc;
+  fill_decode_common(h, &a);
+  const size_t io_bytes = (size_t)items * h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
+  const void* dq = nullptr;
+  void* dout = nullptr;
+  if (int rc = stage_in(h, 0, q, io_bytes, &dq, error_msg)) return rc;
+  if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
+  if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, error_msg)) return rc;
+  a.q = dq;
+  a.out = dout;
+  a.layer_begin = layer_begin;
+  a.n_layers = n_layers;
+  a.batch = batch;
+  a.num_splits = num_splits;
+  a.max_kv_len = max_len;
+  HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream,
+                              h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr));
+  h->timed = h->timing;
+  return stage_out_end(h, 1, out, io_bytes, error_msg);
+}
+
+int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_pos0, int n, const void* q,
+                 void* out, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (int rc = check_layers(h, layer_begin, n_layers, error_msg)) return rc;
+  if (!q || !out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null q or out");
+  if (seq < 0 || seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  if (n < 1 || q_pos0 < 0 || (int64_t)q_pos0 + n > h->cfg.max_tokens)
+    return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "rows [%d, %lld) outside [0, max_tokens=%d]", q_pos0,
+                (long long)q_pos0 + n, h->cfg.max_tokens);
+  for (int l = layer_begin; l < layer_begin + n_layers; ++l)
+    if (q_pos0 + n > h->filled[(size_t)l * h->cfg.max_seqs + seq])
+      return fail(error_msg, MI355_ATTN_OUT_OF_RANGE,
+                  "prefill over rows [0, %d) but only %d rows of layer %d, sequence %d were appended",
+                  q_pos0 + n, h->filled[(size_t)l * h->cfg.max_seqs + seq], l, seq);
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const size_t io_bytes = (size_t)n_layers * n * h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
+  const void* dq = nullptr;
+  void* dout = nullptr;
+  if (int rc = stage_in(h, 0, q, io_bytes, &dq, error_msg)) return rc;
+  if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
+  hipEvent_t e0 = h->timing ? h->ev0 : nullptr, e1 = h->timing ? h->ev1 : nullptr;
+  if (prefill_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim) && !h->rowwise_prefill) {
+    PrefillArgs a{};
+    a.q = dq;
+    a.out = dout;
+    a.cache = h->cache;
+    a.scales = h->scales;
+    a.layer_window = h->d_window;
+    a.geom = h->geom;
+    a.hq = h->cfg.num_q_heads;
+    a.group = h->cfg.num_q_heads / h->cfg.num_kv_heads;
+    a.layer_begin = layer_begin;
+    a.n_layers = n_layers;
+    a.seq = seq;
+    a.q_pos0 = q_pos0;
+    a.n = n;
+    a.scale = h->cfg.scale;
+    a.softcap = h->cfg.softcap;
+    HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
+  } else {
+    // Row-wise path (fp32 and int8 caches): every query row is one decode item
+    // whose key range ends at its own position.
+    if (!decode_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim))
+      return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "prefill: unsupported kv/io dtype pair %d/%d",
+                  h->cfg.kv_dtype, h->cfg.io_dtype);
+    if (h->d_items_cap < (size_t)n) {
+      HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+      if (h->d_items) HIP_OR_RETURN(hipFree(h->d_items));
+      h->d_items = nullptr;
+      h->d_items_cap = 0;
+      HIP_OR_RETURN(hipMalloc(&h->d_items, sizeof(int32_t) * 2 * (size_t)h->cfg.max_tokens));
+      h->d_items_cap = h->cfg.max_tokens;
+    }
+    int32_t* lens = h->d_items;
+    int32_t* seqs = h->d_items + h->d_items_cap;
+    hipLaunchKernelGGL(iota_items_kernel, dim3((n + 255) / 256), dim3(256), 0, h->stream, lens, seqs, n, q_pos0,
+                       seq);
+    HIP_OR_RETURN(hipGetLastError());
+    DecodeArgs a{};
+    fill_decode_common(h, &a);
+    a.q = dq;
+    a.out = dout;
+    a.kv_lens = lens;
+    a.seq_ids = seqs;
+    a.layer_begin = layer_begin;
+    a.n_layers = n_layers;
+    a.batch = n;
+    a.num_splits = 1;
+    a.max_kv_len = q_pos0 + n;
+    HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream, e0, e1));
+  }
+  h->timed = h->timing;
+  return stage_out_end(h, 1, out, io_bytes, error_msg);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mi355_attn_version(void) { return "mi355_attn 0.1 (gfx950)"; }
+
+int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error_msg) {
+  if (out) *out = nullptr;
+  if (!c || !out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null config or out");
+  if (c->struct_size != sizeof(mi355_attn_config))
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "config.struct_size %u != %zu", c->struct_size,
+                sizeof(mi355_attn_config));
+  if (c->num_layers < 1 || c->num_q_heads < 1 || c->num_kv_heads < 1 || c->max_tokens < 1 || c->max_seqs < 1)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "layers, heads, max_tokens and max_seqs must be >= 1");
+  if (c->num_q_heads % c->num_kv_heads)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "num_q_heads %d is not a multiple of num_kv_heads %d",
+                c->num_q_heads, c->num_kv_heads);
+  if (c->num_q_heads / c->num_kv_heads > kMaxGroup)
+    return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "more than %d query heads per KV head", kMaxGroup);
+  if (c->head_dim != 256)
+    return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "head_dim %d (only 256 is built)", c->head_dim);
+  if (c->kv_dtype < MI355_ATTN_F32 || c->kv_dtype > MI355_ATTN_I8 || c->io_dtype < MI355_ATTN_F32 ||
+      c->io_dtype > MI355_ATTN_BF16)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "bad kv_dtype %d or io_dtype %d", c->kv_dtype,
+                c->io_dtype);
+  if (!decode_supported(c->kv_dtype, c->io_dtype, c->head_dim))
+    return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
+                "kv_dtype %d with io_dtype %d (supported: equal f32/f16/bf16, or int8 cache with f16 io)",
+                c->kv_dtype, c->io_dtype);
+  if (c->softcap < 0.f || c->scale < 0.f)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "scale and softcap must be >= 0");
+  if (c->layer_window)
+    for (int l = 0; l < c->num_layers; ++l)
+      if (c->layer_window[l] < 0)
+        return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "layer_window[%d] < 0", l);
+
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1)
+    return fail(error_msg, MI355_ATTN_UNAVAILABLE, "no HIP device");
+  if (c->device < 0 || c->device >= ndev)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "device %d outside [0, %d)", c->device, ndev);
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, c->device) != hipSuccess)
+    return fail(error_msg, MI355_ATTN_UNAVAILABLE, "cannot query device %d", c->device);
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(error_msg, MI355_ATTN_UNAVAILABLE, "device %d is %s; this library is built for gfx950 only",
+                c->device, prop.gcnArchName);
+
+  mi355_attn* h = new (std::nothrow) mi355_attn();
+  if (!h) return fail(error_msg, MI355_ATTN_RESOURCE_EXHAUSTED, "out of host memory");
+  h->cfg = *c;
+  h->cfg.layer_window = nullptr;
+  if (h->cfg.scale == 0.f) h->cfg.scale = 1.0f / sqrtf((float)c->head_dim);
+  h->device = c->device;
+  h->window.assign(c->num_layers, 0);
+  if (c->layer_window) h->window.assign(c->layer_window, c->layer_window + c->num_layers);
+  h->filled.assign((size_t)c->num_layers * c->max_seqs, 0);
+  h->geom.num_layers = c->num_layers;
+  h->geom.max_seqs = c->max_seqs;
+  h->geom.hkv = c->num_kv_heads;
+  h->geom.head_dim = c->head_dim;
+  h->geom.cap = (int32_t)round_up64(c->max_tokens, kTokenAlign);
+  h->geom.esize = dtype_size(c->kv_dtype);
+  h->geom.plane_bytes = (int64_t)h->geom.cap * c->head_dim * h->geom.esize;
+  h->cache_bytes = (uint64_t)h->geom.plane_bytes * 2 * c->num_kv_heads * c->max_seqs * c->num_layers;
+  if (const char* e = getenv("MI355_ATTN_DECODE_WAVES")) h->tuning.waves = atoi(e) == 2 ? 2 : 4;
+  if (const char* e = getenv("MI355_ATTN_DECODE_PIPELINE")) h->tuning.pipeline = atoi(e) != 0;
+
+  auto bail = [&](int code, const char* what, hipError_t e) {
+    int rc = fail(error_msg, code, "%s: %s", what, hipGetErrorString(e));
+    mi355_attn_destroy(h);
+    return rc;
+  };
+  hipError_t e;
+  if ((e = hipSetDevice(h->device)) != hipSuccess) return bail(MI355_ATTN_UNAVAILABLE, "hipSetDevice", e);
+  if (c->own_stream) {
+    if ((e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking)) != hipSuccess)
+      return bail(MI355_ATTN_INTERNAL, "hipStreamCreate", e);
+    h->own_stream = true;
+  } else {
+    h->stream = static_cast<hipStream_t>(c->stream);  // nullptr is the HIP default stream
+  }
+  if ((e = hipMalloc(&h->cache, h->cache_bytes)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "KV cache allocation", e);
+  // Rows that were never written must read as finite numbers: a masked key
+  // still enters P.V with probability 0, and 0 * NaN would poison the output.
+  if ((e = hipMemsetAsync(h->cache, 0, h->cache_bytes, h->stream)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "KV cache clear", e);
+  if (c->kv_dtype == MI355_ATTN_I8) {
+    const size_t nsc = (size_t)c->num_layers * c->max_seqs * 2 * c->num_kv_heads * c->head_dim;
+    if ((e = hipMalloc(&h->scales, nsc * sizeof(float))) != hipSuccess)
+      return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "scale allocation", e);
+    if ((e = hipMemsetAsync(h->scales, 0, nsc * sizeof(float), h->stream)) != hipSuccess)
+      return bail(MI355_ATTN_INTERNAL, "scale clear", e);
+  }
+  if ((e = hipMalloc(&h->d_window, sizeof(int32_t) * c->num_layers)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "window table", e);
+  if ((e = hipMemcpyAsync(h->d_window, h->window.data(), sizeof(int32_t) * c->num_layers, hipMemcpyHostToDevice,
+                          h->stream)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "window upload", e);
+  h->ring_slot_ints = 2 * c->max_seqs;
+  if ((e = hipHostMalloc(&h->h_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "pinned ring", e);
+  if ((e = hipMalloc(&h->d_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "device ring", e);
+  for (int i = 0; i < kRingSlots; ++i)
+    if ((e = hipEventCreateWithFlags(&h->ring_ev[i], hipEventDisableTiming)) != hipSuccess)
+      return bail(MI355_ATTN_INTERNAL, "hipEventCreate", e);
+  if ((e = hipEventCreate(&h->ev0)) != hipSuccess || (e = hipEventCreate(&h->ev1)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "hipEventCreate", e);
+  if ((e = hipStreamSynchronize(h->stream)) != hipSuccess) return bail(MI355_ATTN_INTERNAL, "create sync", e);
+  *out = h;
+  return MI355_ATTN_OK;
+}
+
+void mi355_attn_destroy(mi355_attn* h) {
+  if (!h) return;
+  (void)hipSetDevice(h->device);
+  (void)hipStreamSynchronize(h->stream);
+  if (h->cache) (void)hipFree(h->cache);
+  if (h->scales) (void)hipFree(h->scales);
+  if (h->d_window) (void)hipFree(h->d_window);
+  if (h->ws_acc) (void)hipFree(h->ws_acc);
+  if (h->ws_ml) (void)hipFree(h->ws_ml);
+  if (h->d_ring) (void)hipFree(h->d_ring);
+  if (h->h_ring) (void)hipHostFree(h->h_ring);
+  if (h->d_items) (void)hipFree(h->d_items);
+  for (auto& s : h->stage)
+    if (s) (void)hipFree(s);
+  for (auto& ev : h->ring_ev)
+    if (ev) (void)hipEventDestroy(ev);
+  if (h->ev0) (void)hipEventDestroy(h->ev0);
+  if (h->ev1) (void)hipEventDestroy(h->ev1);
+  if (h->own_stream && h->stream) (void)hipStreamDestroy(h->stream);
+  delete h;
+}
+
+int mi355_attn_kv_append(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos, int32_t n, const void* k,
+                         const void* v, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (seq < 0 || seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  if (n < 0 || pos < 0 || (int64_t)pos + n > h->cfg.max_tokens)
+    return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "rows [%d, %lld) outside [0, max_tokens=%d]", pos,
+                (long long)pos + n, h->cfg.max_tokens);
+  if (n == 0) return MI355_ATTN_OK;
+  if (!k || !v) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null k or v");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const size_t bytes = (size_t)n * h->cfg.num_kv_heads * h->cfg.head_dim * kv_size(h);
+  const void *dk = nullptr, *dv = nullptr;
+  if (int rc = stage_in(h, 2, k, bytes, &dk, error_msg)) return rc;
+  if (int rc = stage_in(h, 3, v, bytes, &dv, error_msg)) return rc;
+  KvCopyArgs a{};
+  a.cache = h->cache;
+  a.geom = h->geom;
+  a.layer = layer;
+  a.seq = seq;
+  a.pos = pos;
+  a.n = n;
+  a.k = const_cast<void*>(dk);
+  a.v = const_cast<void*>(dv);
+  HIP_OR_RETURN(launch_kv_append(a, h->stream));
+  if (h->cfg.host_io) HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  int32_t& f = h->filled[(size_t)layer * h->cfg.max_seqs + seq];
+  f = std::max(f, pos + n);
+  return MI355_ATTN_OK;
+}
+
+int mi355_attn_kv_set_scales(mi355_attn* h, int32_t layer, int32_t seq, const float* k_scale,
+                             const float* v_scale, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (h->cfg.kv_dtype != MI355_ATTN_I8)
+    return fail(error_msg, MI355_ATTN_FAILED_PRECONDITION, "scales apply to an int8 cache only");
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (seq < 0 || seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  if (!k_scale || !v_scale) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null scales");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const size_t n = (size_t)h->cfg.num_kv_heads * h->cfg.head_dim;
+  const hipMemcpyKind kind = h->cfg.host_io ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
+  HIP_OR_RETURN(hipMemcpyAsync(h->scales + h->geom.scale_offset(layer, seq, 0, 0), k_scale, n * sizeof(float), kind,
+                               h->stream));
+  HIP_OR_RETURN(hipMemcpyAsync(h->scales + h->geom.scale_offset(layer, seq, 1, 0), v_scale, n * sizeof(float), kind,
+                               h->stream));
+  if (h->cfg.host_io) HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  return MI355_ATTN_OK;
+}
+
+int mi355_attn_kv_read(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos, int32_t n, void* k_out, void* v_out,
+                       char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (seq < 0 || seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  if (n < 0 || pos < 0 || (int64_t)pos + n > h->cfg.max_tokens)
+    return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "rows [%d, %lld) outside [0, max_tokens=%d]", pos,
+                (long long)pos + n, h->cfg.max_tokens);
+  if (n == 0) return MI355_ATTN_OK;
+  if (!k_out || !v_out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null k_out or v_out");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const size_t bytes = (size_t)n * h->cfg.num_kv_heads * h->cfg.head_dim * kv_size(h);
+  void *dk = nullptr, *dv = nullptr;
+  if (int rc = stage_out_begin(h, 2, k_out, bytes, &dk, error_msg)) return rc;
+  if (int rc = stage_out_begin(h, 3, v_out, bytes, &dv, error_msg)) return rc;
+  KvCopyArgs a{};
+  a.cache = h->cache;
+  a.geom = h->geom;
+  a.layer = layer;
+  a.seq = seq;
+  a.pos = pos;
+  a.n = n;
+  a.k = dk;
+  a.v = dv;
+  HIP_OR_RETURN(launch_kv_read(a, h->stream));
+  if (int rc = stage_out_end(h, 2, k_out, bytes, error_msg)) return rc;
+  return stage_out_end(h, 3, v_out, bytes, error_msg);
+}
+
+int mi355_attn_prefill(mi355_attn* h, int32_t layer, int32_t seq, int32_t q_pos0, int32_t n, const void* q,
+                       void* out, char** error_msg) {
+  return prefill_impl(h, layer, 1, seq, q_pos0, n, q, out, error_msg);
+}
+
+int mi355_attn_prefill_layers(mi355_attn* h, int32_t layer_begin, int32_t n_layers, int32_t seq, int32_t q_pos0,
+                              int32_t n, const void* q, void* out, char** error_msg) {
+  return prefill_impl(h, layer_begin, n_layers, seq, q_pos0, n, q, out, error_msg);
+}
+
+int mi355_attn_decode(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens, int32_t batch,
+                      const void* q, void* out, int32_t num_splits, char** error_msg) {
+  return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg);
+}
+
+int mi355_attn_decode_layers(mi355_attn* h, int32_t layer_begin, int32_t n_layers, const int32_t* seq_ids,
+                             const int32_t* kv_lens, int32_t batch, const void* q, void* out, int32_t num_splits,
+                             char** error_msg) {
+  return decode_impl(h, layer_begin, n_layers, seq_ids, kv_lens, batch, q, out, num_splits, error_msg);
+}
+
+int mi355_attn_reset(mi355_attn* h, int32_t seq, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  for (int l = 0; l < h->cfg.num_layers; ++l)
+    for (int s = 0; s < h->cfg.max_seqs; ++s)
+      if (seq < 0 || s == seq) h->filled[(size_t)l * h->cfg.max_seqs + s] = 0;
+  return MI355_ATTN_OK;
+}
+
+int mi355_attn_sync(mi355_attn* h, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  return MI355_ATTN_OK;
+}
+
+void* mi355_attn_stream(mi355_attn* h) { return h ? h->stream : nullptr; }
+
+int mi355_attn_set_timing(mi355_attn* h, int32_t enabled) {
+  if (!h) return MI355_ATTN_INVALID_ARGUMENT;
+  h->timing = enabled != 0;
+  h->timed = false;
+  return MI355_ATTN_OK;
+}
+
+float mi355_attn_last_kernel_ms(mi355_attn* h) {
+  if (!h || !h->timed) return -1.f;
+  if (hipEventSynchronize(h->ev1) != hipSuccess) return -1.f;
+  float ms = -1.f;
+  if (hipEventElapsedTime(&ms, h->ev0, h->ev1) != hipSuccess) return -1.f;
+  return ms;
+}
+
+int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
+  if (!h || !name) return MI355_ATTN_INVALID_ARGUMENT;
+  if (!strcmp(name, "decode_waves")) {
+    if (value != 2 && value != 4) return MI355_ATTN_INVALID_ARGUMENT;
+    h->tuning.waves = value;
+  } else if (!strcmp(name, "decode_pipeline")) {
+    h->tuning.pipeline = value != 0;
+  } else if (!strcmp(name, "rowwise_prefill")) {
+    h->rowwise_prefill = value != 0;
+  } else {
+    return MI355_ATTN_INVALID_ARGUMENT;
+  }
+  return MI355_ATTN_OK;
+}
+
+uint64_t mi355_attn_cache_bytes(const mi355_attn* h) { return h ? h->cache_bytes : 0; }
+
+}  // extern "C"

@@ -338,3 +338,31 @@ def rel_err(a, b) -> float:
     b = np.asarray(b, dtype=np.float64)
     den = np.abs(b).max()
     return float(np.abs(a - b).max() / (den if den > 0 else 1.0))
+
+
+def l2_rel_err(a, b) -> float:
+    """||a-b||_2 / ||b||_2 per output tensor."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    den = np.sqrt((b * b).sum())
+    return float(np.sqrt(((a - b) ** 2).sum()) / (den if den > 0 else 1.0))
+
+
+def half_ulp_bf16(x) -> np.ndarray:
+    """Largest error that rounding x to bfloat16 (8 significant bits) can add."""
+    x = np.abs(np.asarray(x, dtype=np.float64))
+    _, ex = np.frexp(x)  # x = m * 2**ex, m in [0.5, 1)
+    return np.where(x > 0, np.ldexp(1.0, ex - 9), 0.0)
+
+
+def rel_err_beyond_bf16_rounding(a, b) -> float:
+    """Norm-wise relative error after discounting, element by element, the
+    half-ulp that storing the result as bfloat16 must cost. A bfloat16 output
+    cannot meet a 2e-3 max-norm bound by format alone (half an ulp is up to
+    2^-8 = 3.9e-3 of the element), so bf16 results are judged by this figure
+    and by l2_rel_err."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    excess = np.maximum(np.abs(a - b) - half_ulp_bf16(b), 0.0)
+    den = np.abs(b).max()
+    return float(excess.max() / (den if den > 0 else 1.0))

@@ -1,0 +1,468 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on
+identical seeded inputs.
+
+Tolerances (norm-wise relative error max|a-b| / max|ref| per output tensor):
+fp32 <= 1e-5, fp16 / bf16 / int8-KV <= 2e-3.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from __graft_entry__ import load_package  # noqa: E402
+from oracle import attn_oracle as orc  # noqa: E402
+from oracle import c_oracle  # noqa: E402
+
+A = load_package().attn
+DEV = "cuda:0"
+TOL = {A.F32: 1e-5, A.F16: 2e-3, A.BF16: 2e-3, A.I8: 2e-3}
+TDT = {A.F32: torch.float32, A.F16: torch.float16, A.BF16: torch.bfloat16, A.I8: torch.int8}
+D = 256
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def err_of(got, ref, dt):
+    """The figure held against TOL[dt]. fp32 / fp16 / int8-KV (fp16 output):
+    max|a-b| / max|ref|. bf16 output: the same after discounting the half-ulp of
+    the bfloat16 output format (which alone can reach 3.9e-3 of an element), and
+    the L2-relative error must stay under the same 2e-3."""
+    if dt == A.BF16:
+        l2 = orc.l2_rel_err(got, ref)
+        assert l2 < TOL[dt], f"bf16 L2-relative error {l2:.3e}"
+        return orc.rel_err_beyond_bf16_rounding(got, ref)
+    return orc.rel_err(got, ref)
+
+
+def make(num_layers, hq, hkv, max_tokens, max_seqs, kv, io=None, **kw):
+    io = (A.F16 if kv == A.I8 else kv) if io is None else io
+    return A.Attn(num_layers, hq, hkv, D, max_tokens, max_seqs, kv, io,
+                  stream=torch.cuda.current_stream().cuda_stream, **kw)
+
+
+def dev(x, dt):
+    """numpy fp32 -> device tensor of dtype dt, and the rounded values back as fp32 numpy."""
+    t = torch.from_numpy(np.ascontiguousarray(x)).to(DEV).to(TDT[dt]).contiguous()
+    return t, t.float().cpu().numpy()
+
+
+def gen(seed, *shape):
+    return np.random.default_rng(seed).standard_normal(shape).astype(np.float32)
+
+
+# ------------------------------------------------------------------ cache layout
+@pytest.mark.parametrize("kv", [A.F32, A.F16, A.BF16, A.I8])
+def test_kv_roundtrip_bit_exact(kv):
+    say(f"kv_roundtrip kv={kv}")
+    hkv, cap = 2, 300
+    with make(2, 4, hkv, cap, 3, kv) as at:
+        rng = np.random.default_rng(kv)
+        if kv == A.I8:
+            k = torch.from_numpy(rng.integers(-127, 128, (cap, hkv, D), dtype=np.int8)).to(DEV)
+            v = torch.from_numpy(rng.integers(-127, 128, (cap, hkv, D), dtype=np.int8)).to(DEV)
+        else:
+            k, _ = dev(gen(1, cap, hkv, D), kv)
+            v, _ = dev(gen(2, cap, hkv, D), kv)
+        # three appends with ragged boundaries, into layer 1 / sequence 2
+        for lo, hi in ((0, 5), (5, 133), (133, cap)):
+            at.kv_append(1, 2, lo, k[lo:hi].contiguous(), v[lo:hi].contiguous())
+        ko, vo = torch.zeros_like(k), torch.zeros_like(v)
+        at.kv_read(1, 2, 0, cap, ko, vo)
+        torch.cuda.synchronize()
+        assert torch.equal(ko.view(torch.uint8), k.view(torch.uint8))
+        assert torch.equal(vo.view(torch.uint8), v.view(torch.uint8))
+        # an unaligned window of rows
+        k2, v2 = torch.zeros_like(k[:77]), torch.zeros_like(v[:77])
+        at.kv_read(1, 2, 41, 77, k2, v2)
+        torch.cuda.synchronize()
+        assert torch.equal(k2.view(torch.uint8), k[41:118].view(torch.uint8))
+        assert torch.equal(v2.view(torch.uint8), v[41:118].view(torch.uint8))
+        # other (layer, sequence) planes stay zero
+        at.kv_append(0, 0, 0, k[:1].contiguous(), v[:1].contiguous())
+        at.kv_read(0, 1, 0, cap, ko, vo)
+        torch.cuda.synchronize()
+        assert int(ko.view(torch.uint8).count_nonzero()) == 0 and int(vo.view(torch.uint8).count_nonzero()) == 0
+
+
+# ------------------------------------------------------------------ decode
+def run_decode(at, kv, q, kvs, lens, layer=0, num_splits=0, seq_ids=None, window=0, softcap=0.0, scale=None,
+               scales=None):
+    """q [B,Hq,D] fp32 numpy; kvs list of (k, v) fp32 numpy [L,Hkv,D] already rounded (or int8 + scales)."""
+    io = A.F16 if kv == A.I8 else kv
+    qd, qr = dev(q, io)
+    out = torch.empty_like(qd)
+    at.decode(layer, lens, qd, out, seq_ids=seq_ids, num_splits=num_splits)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    scale = D ** -0.5 if scale is None else scale
+    errs = []
+    for b, n in enumerate(lens):
+        k, v = kvs[b]
+        if softcap:
+            ref = orc.decode_attn(qr[b], k, v, scale, n, window=window, softcap=softcap)
+        else:
+            ref = c_oracle.sdpa_f64(qr[b:b + 1], k, v, scale, q_pos0=n - 1, window=window, kv_len=n)[0]
+        errs.append(err_of(got[b], ref, kv))
+    return max(errs), got
+
+
+def fill_seq(at, kv, layer, seq, k, v):
+    """Appends fp32 numpy rows (rounded to the cache dtype); returns the rounded fp32 values."""
+    kd, kr = dev(k, kv)
+    vd, vr = dev(v, kv)
+    at.kv_append(layer, seq, 0, kd, vd)
+    return kr, vr
+
+
+def test_decode_c1_fp32_all_variants():
+    # config 1: B1, Hq4/Hkv1, L1024, fp32
+    seed = orc.SEED_BASE + 0
+    q = gen(seed, 1, 4, D)
+    k, v = gen(seed + 100, 1024, 1, D), gen(seed + 200, 1024, 1, D)
+    with make(1, 4, 1, 1024, 1, A.F32) as at:
+        kr, vr = fill_seq(at, A.F32, 0, 0, k, v)
+        for waves in (4, 2):
+            for pipe in (0, 1):
+                at.set_option("decode_waves", waves)
+                at.set_option("decode_pipeline", pipe)
+                for ns in (1, 2, 16, 0):
+                    err, _ = run_decode(at, A.F32, q, [(kr, vr)], [1024], num_splits=ns)
+                    say(f"C1 fp32 waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
+                    assert err < TOL[A.F32]
+
+
+@pytest.mark.parametrize("kv", [A.F16, A.BF16])
+def test_decode_c3_split16(kv):
+    seed = orc.SEED_BASE + 2
+    q = gen(seed, 1, 8, D)
+    k, v = gen(seed + 100, 4096, 2, D), gen(seed + 200, 4096, 2, D)
+    with make(1, 8, 2, 4096, 1, kv) as at:
+        kr, vr = fill_seq(at, kv, 0, 0, k, v)
+        for waves in (4, 2):
+            for pipe in (0, 1):
+                at.set_option("decode_waves", waves)
+                at.set_option("decode_pipeline", pipe)
+                for ns in (16, 1, 5):
+                    err, _ = run_decode(at, kv, q, [(kr, vr)], [4096], num_splits=ns)
+                    say(f"C3 kv={kv} waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
+                    assert err < TOL[kv]
+
+
+@pytest.mark.parametrize("kv", [A.F32, A.F16, A.BF16])
+def test_decode_ragged_lengths_and_seq_ids(kv):
+    lens = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 300, 700]
+    rng = np.random.default_rng(7)
+    slots = list(rng.permutation(len(lens) + 2)[: len(lens)])  # scattered cache slots
+    with make(1, 8, 2, 700, len(lens) + 2, kv) as at:
+        kvs = []
+        for b, n in enumerate(lens):
+            kr, vr = fill_seq(at, kv, 0, int(slots[b]), gen(100 + b, n, 2, D), gen(200 + b, n, 2, D))
+            kvs.append((kr, vr))
+        q = gen(5, len(lens), 8, D)
+        for ns in (1, 3, 8):
+            err, _ = run_decode(at, kv, q, kvs, lens, num_splits=ns, seq_ids=slots)
+            say(f"ragged kv={kv} splits={ns}: rel_err={err:.3e}")
+            assert err < TOL[kv]
+        # shorter views of the same caches (stale rows behind kv_len must stay invisible)
+        short = [max(1, n // 2) for n in lens]
+        err, _ = run_decode(at, kv, q, kvs, short, num_splits=4, seq_ids=slots)
+        say(f"ragged-short kv={kv}: rel_err={err:.3e}")
+        assert err < TOL[kv]
+
+
+@pytest.mark.parametrize("kv", [A.F32, A.F16])
+def test_decode_sliding_window_layers(kv):
+    windows = [0, 512, 1, 37, 64, 100]
+    L = 1500
+    with make(len(windows), 4, 1, L, 1, kv, layer_window=windows) as at:
+        k, v = gen(11, L, 1, D), gen(12, L, 1, D)
+        q = gen(13, 1, 4, D)
+        for layer, w in enumerate(windows):
+            kr, vr = fill_seq(at, kv, layer, 0, k, v)
+            for n in (1, 36, 37, 38, 511, 512, 513, 1024, 1500):
+                for ns in (1, 4):
+                    err, _ = run_decode(at, kv, q, [(kr, vr)], [n], layer=layer, num_splits=ns, window=w)
+                    assert err < TOL[kv], (layer, w, n, ns, err)
+            say(f"window kv={kv} layer={layer} W={w}: ok")
+
+
+def test_decode_int8_kv():
+    # config 5 reduced: 3 sequences, per-(head, channel) scales per sequence
+    lens = [4096, 1000, 65]
+    with make(1, 8, 2, 4096, 3, A.I8) as at:
+        kvs = []
+        for b, n in enumerate(lens):
+            k, v = gen(300 + b, n, 2, D), gen(400 + b, n, 2, D)
+            kq, ks = orc.quantize_kv_int8(k)
+            vq, vs = orc.quantize_kv_int8(v)
+            at.kv_append(0, b, 0, torch.from_numpy(kq).to(DEV), torch.from_numpy(vq).to(DEV))
+            at.kv_set_scales(0, b, torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
+            kvs.append((orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs)))
+        q = gen(9, len(lens), 8, D)
+        for waves in (4, 2):
+            for pipe in (0, 1):
+                at.set_option("decode_waves", waves)
+                at.set_option("decode_pipeline", pipe)
+                for ns in (1, 16):
+                    err, _ = run_decode(at, A.I8, q, kvs, lens, num_splits=ns)
+                    say(f"int8 waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
+                    assert err < TOL[A.I8]
+
+
+def test_decode_softcap_and_scale():
+    with make(1, 4, 2, 256, 1, A.F32, scale=0.11, softcap=3.0) as at:
+        kr, vr = fill_seq(at, A.F32, 0, 0, gen(21, 200, 2, D), gen(22, 200, 2, D))
+        q = 3.0 * gen(23, 1, 4, D)
+        err, _ = run_decode(at, A.F32, q, [(kr, vr)], [200], num_splits=2, softcap=3.0, scale=0.11)
+        say(f"softcap fp32: rel_err={err:.3e}")
+        assert err < 2e-5  # tanh goes through the device libm
+
+
+def test_decode_closed_forms_on_device():
+    # identical keys -> mean of values; constant values -> constant output
+    L = 333
+    with make(1, 8, 2, 512, 1, A.F16) as at:
+        k = np.broadcast_to(gen(31, 1, 2, D), (L, 2, D)).copy()
+        v = gen(32, L, 2, D)
+        kr, vr = fill_seq(at, A.F16, 0, 0, k, v)
+        qd, _ = dev(gen(33, 1, 8, D), A.F16)
+        out = torch.empty_like(qd)
+        at.decode(0, [L], qd, out, num_splits=3)
+        torch.cuda.synchronize()
+        exp = np.repeat(vr.astype(np.float64).mean(axis=0), 4, axis=0)
+        assert orc.rel_err(out.float().cpu().numpy()[0], exp) < TOL[A.F16]
+        kr, vr = fill_seq(at, A.F16, 0, 0, gen(34, L, 2, D), np.full((L, 2, D), 0.75, np.float32))
+        at.decode(0, [L], qd, out, num_splits=3)
+        torch.cuda.synchronize()
+        assert np.abs(out.float().cpu().numpy() - 0.75).max() < 1e-3
+
+
+def test_decode_layers_equals_per_layer_calls():
+    nl, B, L = 3, 4, 500
+    with make(nl, 8, 2, 512, B, A.F16, layer_window=[0, 128, 0]) as at:
+        for layer in range(nl):
+            for b in range(B):
+                fill_seq(at, A.F16, layer, b, gen(50 + 10 * layer + b, L, 2, D), gen(90 + 10 * layer + b, L, 2, D))
+        lens = [500, 77, 256, 1]
+        qd, _ = dev(gen(41, nl, B, 8, D), A.F16)
+        out_all = torch.empty_like(qd)
+        at.decode(0, lens, qd, out_all, num_splits=4, n_layers=nl)
+        outs = torch.empty_like(qd)
+        for layer in range(nl):
+            at.decode(layer, lens, qd[layer], outs[layer], num_splits=4)
+        torch.cuda.synchronize()
+        assert torch.equal(out_all, outs)
+
+
+# ------------------------------------------------------------------ prefill
+def run_prefill(at, dt, q, kr, vr, q_pos0, window, layer=0, rowwise=False, scale=None):
+    qd, qr = dev(q, dt)
+    out = torch.empty_like(qd)
+    at.set_option("rowwise_prefill", int(rowwise))
+    at.prefill(layer, 0, q_pos0, q.shape[0], qd, out)
+    torch.cuda.synchronize()
+    scale = D ** -0.5 if scale is None else scale
+    ref = c_oracle.sdpa_f64(qr, kr, vr, scale, q_pos0=q_pos0, window=window, kv_len=q_pos0 + q.shape[0])
+    return err_of(out.float().cpu().numpy(), ref, dt), out
+
+
+@pytest.mark.parametrize("dt", [A.BF16, A.F16])
+@pytest.mark.parametrize("hq,hkv", [(4, 1), (8, 2), (2, 2), (2, 1), (3, 1)])
+def test_prefill_small_shapes(dt, hq, hkv):
+    windows = [0, 40, 1, 33]
+    L = 400
+    with make(len(windows), hq, hkv, L, 1, dt, layer_window=windows) as at:
+        k, v = gen(61, L, hkv, D), gen(62, L, hkv, D)
+        for layer, w in enumerate(windows):
+            kr, vr = fill_seq(at, dt, layer, 0, k, v)
+            for q_pos0, n in ((0, 1), (0, 31), (0, 32), (0, 33), (0, 100), (0, 257), (70, 64), (129, 200), (399, 1)):
+                q = gen(1000 + n + q_pos0, n, hq, D)
+                err, out = run_prefill(at, dt, q, kr, vr, q_pos0, w, layer=layer)
+                assert err < TOL[dt], (hq, hkv, w, q_pos0, n, err)
+                err_r, out_r = run_prefill(at, dt, q, kr, vr, q_pos0, w, layer=layer, rowwise=True)
+                assert err_r < TOL[dt], ("rowwise", hq, hkv, w, q_pos0, n, err_r)
+        say(f"prefill small dt={dt} hq={hq} hkv={hkv}: ok")
+
+
+def test_prefill_c2_full_size_local_and_global():
+    # config 2: 1024-token chunk, Hq4/Hkv1, bf16; one local (W=512) and one global layer
+    seed = orc.SEED_BASE + 1
+    with make(2, 4, 1, 1024, 1, A.BF16, layer_window=[512, 0]) as at:
+        for layer, w in ((0, 512), (1, 0)):
+            q = gen(seed + layer, 1024, 4, D)
+            kr, vr = fill_seq(at, A.BF16, layer, 0, gen(seed + 10 + layer, 1024, 1, D), gen(seed + 20 + layer, 1024, 1, D))
+            err, _ = run_prefill(at, A.BF16, q, kr, vr, 0, w, layer=layer)
+            say(f"C2 bf16 layer window={w}: rel_err={err:.3e}")
+            assert err < TOL[A.BF16]
+
+
+def test_prefill_chunked_equals_one_shot_and_layers_call():
+    # two chunks (600 + 424) over a growing cache == one 1024 chunk; prefill_layers == per-layer calls
+    nl = 2
+    with make(nl, 4, 1, 1024, 1, A.BF16, layer_window=[512, 0]) as at:
+        qd, _ = dev(gen(71, nl, 1024, 4, D), A.BF16)
+        for layer in range(nl):
+            kd, _ = dev(gen(72 + layer, 1024, 1, D), A.BF16)
+            vd, _ = dev(gen(75 + layer, 1024, 1, D), A.BF16)
+            at.kv_append(layer, 0, 0, kd, vd)
+        one = torch.empty_like(qd)
+        at.prefill(0, 0, 0, 1024, qd, one, n_layers=nl)
+        per = torch.empty_like(qd)
+        two = torch.empty_like(qd)
+        for layer in range(nl):
+            at.prefill(layer, 0, 0, 1024, qd[layer], per[layer])
+            at.prefill(layer, 0, 0, 600, qd[layer, :600].contiguous(), two[layer, :600])
+            at.prefill(layer, 0, 600, 424, qd[layer, 600:].contiguous(), two[layer, 600:])
+        torch.cuda.synchronize()
+        assert torch.equal(one, per)
+        # different tile alignment changes the summation order, not the result
+        assert orc.rel_err(two.float().cpu().numpy(), one.float().cpu().numpy()) < TOL[A.BF16]
+
+
+def test_prefill_rowwise_fp32_and_int8():
+    L = 200
+    with make(1, 4, 1, 256, 1, A.F32, layer_window=[50]) as at:
+        kr, vr = fill_seq(at, A.F32, 0, 0, gen(81, L, 1, D), gen(82, L, 1, D))
+        err, _ = run_prefill(at, A.F32, gen(83, 150, 4, D), kr, vr, 50, 50)
+        say(f"prefill fp32 rowwise: rel_err={err:.3e}")
+        assert err < TOL[A.F32]
+    with make(1, 8, 2, 256, 1, A.I8) as at:
+        k, v = gen(84, L, 2, D), gen(85, L, 2, D)
+        kq, ks = orc.quantize_kv_int8(k)
+        vq, vs = orc.quantize_kv_int8(v)
+        at.kv_append(0, 0, 0, torch.from_numpy(kq).to(DEV), torch.from_numpy(vq).to(DEV))
+        at.kv_set_scales(0, 0, torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
+        err, _ = run_prefill(at, A.F16, gen(86, L, 8, D), orc.dequantize_kv_int8(kq, ks),
+                             orc.dequantize_kv_int8(vq, vs), 0, 0)
+        say(f"prefill int8 rowwise: rel_err={err:.3e}")
+        assert err < TOL[A.I8]
+
+
+# ------------------------------------------------------------------ full-size configs 4 and 5
+def test_c4_batched_ragged_full_size():
+    rng = orc.config_rng(3)
+    lens = [int(x) for x in rng.integers(256, 4097, size=64)]
+    with make(1, 8, 2, 4096, 64, A.F16) as at:
+        kvs = []
+        for b, n in enumerate(lens):
+            g = torch.Generator(device=DEV).manual_seed(1000 + b)
+            kd = torch.randn((n, 2, D), generator=g, device=DEV, dtype=torch.float32).half()
+            vd = torch.randn((n, 2, D), generator=g, device=DEV, dtype=torch.float32).half()
+            at.kv_append(0, b, 0, kd, vd)
+            kvs.append((kd.float().cpu().numpy(), vd.float().cpu().numpy()))
+        q = gen(orc.SEED_BASE + 3, 64, 8, D)
+        for ns in (16, 0):
+            err, _ = run_decode(at, A.F16, q, kvs, lens, num_splits=ns)
+            say(f"C4 full splits={ns}: rel_err={err:.3e}")
+            assert err < TOL[A.F16]
+
+
+def test_c5_int8_full_size_properties():
+    # 32 sequences x 4096 int8; oracle on 4 of them, linearity in V on all
+    B, L = 32, 4096
+    with make(1, 8, 2, L, B, A.I8) as at:
+        rng = np.random.default_rng(orc.SEED_BASE + 4)
+        check = {0, 7, 19, 31}
+        kvs = {}
+        for b in range(B):
+            k = rng.standard_normal((L, 2, D)).astype(np.float32)
+            v = rng.standard_normal((L, 2, D)).astype(np.float32)
+            kq, ks = orc.quantize_kv_int8(k)
+            vq, vs = orc.quantize_kv_int8(v)
+            at.kv_append(0, b, 0, torch.from_numpy(kq).to(DEV), torch.from_numpy(vq).to(DEV))
+            at.kv_set_scales(0, b, torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
+            if b in check:
+                kvs[b] = (orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs))
+        q = gen(orc.SEED_BASE + 40, B, 8, D)
+        qd, qr = dev(q, A.F16)
+        out = torch.empty_like(qd)
+        at.decode(0, [L] * B, qd, out, num_splits=8)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        for b in sorted(check):
+            ref = c_oracle.sdpa_f64(qr[b:b + 1], kvs[b][0], kvs[b][1], D ** -0.5, q_pos0=L - 1)[0]
+            err = orc.rel_err(got[b], ref)
+            say(f"C5 full seq {b}: rel_err={err:.3e}")
+            assert err < TOL[A.I8]
+        assert np.isfinite(got).all()
+        # size-independent property on all 32 sequences: doubling every V scale doubles the output
+        for b in range(B):
+            ks = torch.full((2, D), 0.02, device=DEV)
+            at.kv_set_scales(0, b, ks, ks)
+        o1 = torch.empty_like(qd)
+        at.decode(0, [L] * B, qd, o1, num_splits=8)
+        for b in range(B):
+            at.kv_set_scales(0, b, torch.full((2, D), 0.02, device=DEV), torch.full((2, D), 0.04, device=DEV))
+        o2 = torch.empty_like(qd)
+        at.decode(0, [L] * B, qd, o2, num_splits=8)
+        torch.cuda.synchronize()
+        assert orc.rel_err(o2.float().cpu().numpy(), 2.0 * o1.float().cpu().numpy()) < 1e-3
+
+
+# ------------------------------------------------------------------ error behaviour (no kernel is launched)
+def test_error_codes():
+    with pytest.raises(A.AttnError) as e:
+        A.Attn(1, 3, 2, D, 16, 1, A.F16, A.F16)
+    assert e.value.code == A.INVALID_ARGUMENT
+    with pytest.raises(A.AttnError) as e:
+        A.Attn(1, 4, 1, 128, 16, 1, A.F16, A.F16)
+    assert e.value.code == A.UNIMPLEMENTED
+    with make(1, 4, 1, 100, 2, A.F16) as at:
+        kd, _ = dev(gen(1, 10, 1, D), A.F16)
+        qd, _ = dev(gen(2, 1, 4, D), A.F16)
+        out = torch.empty_like(qd)
+        with pytest.raises(A.AttnError) as e:
+            at.kv_append(0, 0, 95, kd, kd)
+        assert e.value.code == A.OUT_OF_RANGE
+        with pytest.raises(A.AttnError) as e:
+            at.kv_append(1, 0, 0, kd, kd)
+        assert e.value.code == A.INVALID_ARGUMENT
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [5], qd, out)  # nothing appended yet
+        assert e.value.code == A.OUT_OF_RANGE
+        at.kv_append(0, 0, 0, kd, kd)
+        at.decode(0, [10], qd, out)
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [11], qd, out)
+        assert e.value.code == A.OUT_OF_RANGE
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [0], qd, out)
+        assert e.value.code == A.OUT_OF_RANGE
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [1, 1, 1], qd, out)  # batch > max_seqs
+        assert e.value.code == A.INVALID_ARGUMENT
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [5], qd, out, seq_ids=[2])
+        assert e.value.code == A.INVALID_ARGUMENT
+        with pytest.raises(A.AttnError) as e:
+            at.kv_set_scales(0, 0, qd, qd)
+        assert e.value.code == A.FAILED_PRECONDITION
+        at.reset()
+        with pytest.raises(A.AttnError) as e:
+            at.decode(0, [10], qd, out)  # rows forgotten by reset
+        assert e.value.code == A.OUT_OF_RANGE
+        torch.cuda.synchronize()
+
+
+def test_host_io_mode():
+    # host pointers at the boundary, as the reference's host TensorBuffers
+    L = 130
+    k, v, q = gen(91, L, 1, D), gen(92, L, 1, D), gen(93, L, 4, D)
+    with A.Attn(1, 4, 1, D, 256, 1, A.F32, A.F32, host_io=True) as at:
+        at.kv_append(0, 0, 0, k, v)
+        out = np.zeros_like(q)
+        at.prefill(0, 0, 0, L, q, out)
+        ref = orc.sdpa(q, k, v, D ** -0.5)
+        assert orc.rel_err(out, ref) < TOL[A.F32]
+        dec = np.zeros((1, 4, D), np.float32)
+        at.decode(0, [L], q[L - 1:L].copy(), dec, num_splits=2)
+        assert orc.rel_err(dec[0], ref[L - 1]) < TOL[A.F32]
