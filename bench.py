@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+One "step" is one pass of decode attention over the KV caches of all 30 layers
+of a Gemma3n-E2B-shaped model at 4096 context (config 3 of BASELINE.json:
+batch 1, 8 query heads / 2 KV heads, head_dim 256, fp16 cache, 16 split-KV
+partitions merged by log-sum-exp), issued as one multi-layer launch plus the
+merge pass. A single layer is only 8 MiB and would sit in cache, so each step
+streams a different set of 30 layer caches out of 4 (1 GiB in total): reads
+come from HBM, not from L2 / Infinity Cache.
+
+Prints ONE JSON line. `value` is algorithmic bytes per step / wall time per
+step with all inputs resident in HBM. `roofline` prices the decode attention
+kernel alone (HIP events around each launch, on the stream it runs on) against
+the 8 TB/s HBM peak. `prefill` is the 26-layer, 1024-token bf16 prefill of
+config 2 in one launch, priced against the 2.5 PFLOP/s dense bf16 MFMA peak.
+`cpu_baseline` times the C restatement of the reference CPU op order
+(oracle/attn_oracle.c) on a bounded sample of the same decode workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+D = 256
+METRIC = "decode-attn HBM GB/s (% of 8 TB/s) + prefill-attn TFLOP/s, Gemma3n-E2B shape"
+
+# HBM bytes per decode launch of the headline workload, from
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script, each
+# scaled by what the same counter reads for a plain copy of known size
+# (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def fill_cache(at, torch, layers, seqs_lens, hkv, dtype, seed):
+    """Appends N(0,1) rows (generated on the GPU) to every (layer, sequence)."""
+    g = torch.Generator(device="cuda:0").manual_seed(seed)
+    for layer in range(layers):
+        for seq, n in enumerate(seqs_lens):
+            k = torch.randn((n, hkv, D), generator=g, device="cuda:0", dtype=torch.float32).to(dtype)
+            v = torch.randn((n, hkv, D), generator=g, device="cuda:0", dtype=torch.float32).to(dtype)
+            at.kv_append(layer, seq, 0, k, v)
+
+
+def time_steps(torch, step_fn, steps, warmup):
+    for i in range(warmup):
+        step_fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step_fn(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_ms(torch, at, step_fn, launches, first):
+    """Average duration of the attention kernel itself over `launches` calls."""
+    at.set_timing(True)
+    total = 0.0
+    for i in range(launches):
+        step_fn(first + i)
+        total += at.last_kernel_ms()
+    at.set_timing(False)
+    return total / launches
+
+
+def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, ctx=4096):
+    hq, hkv = 8, 2
+    stream = torch.cuda.current_stream().cuda_stream
+    at = A.Attn(layers * rotation, hq, hkv, D, ctx, 1, A.F16, A.F16, stream=stream)
+    fill_cache(at, torch, layers * rotation, [ctx], hkv, torch.float16, seed=0xC0FFEE + 2)
+    q = torch.randn((rotation, layers, 1, hq, D), device="cuda:0", dtype=torch.float32).half()
+    out = torch.empty_like(q)
+    lens = A._i32_array([ctx])
+
+    def step(i):
+        r = i % rotation
+        at.decode(r * layers, lens, q[r], out[r], num_splits=splits, n_layers=layers, batch=1)
+
+    sec = time_steps(torch, step, steps, warmup)
+    kms = kernel_ms(torch, at, step, min(steps, 50), warmup + steps)
+    # algorithmic bytes: K and V once, Q and O once (no partials, no padding)
+    per_layer = ctx * hkv * D * 2 * 2 + 2 * hq * D * 2
+    step_bytes = per_layer * layers
+    # single layer, cache resident: latency figure only
+    def step1(i):
+        at.decode(0, lens, q[0, 0], out[0, 0], num_splits=splits, batch=1)
+    lat = time_steps(torch, step1, 200, 20)
+    at.close()
+    return {"sec_per_step": sec, "kernel_ms": kms, "step_bytes": step_bytes, "layers": layers,
+            "single_layer_latency_us": lat * 1e6, "tokens_per_s": 1.0 / sec}
+
+
+def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits):
+    """Single-layer batched decode (configs 4 and 5), rotating over `rotation` layers."""
+    hq, hkv = 8, 2
+    B = len(lens)
+    stream = torch.cuda.current_stream().cuda_stream
+    at = A.Attn(rotation, hq, hkv, D, 4096, B, kv, A.F16, stream=stream)
+    g = torch.Generator(device="cuda:0").manual_seed(0xC0FFEE + (3 if kv == A.F16 else 4))
+    for layer in range(rotation):
+        for b, n in enumerate(lens):
+            if kv == A.I8:
+                k = torch.randint(-127, 128, (n, hkv, D), generator=g, device="cuda:0", dtype=torch.int8)
+                v = torch.randint(-127, 128, (n, hkv, D), generator=g, device="cuda:0", dtype=torch.int8)
+                sc = torch.rand((hkv, D), generator=g, device="cuda:0") * 0.02 + 0.02
+                at.kv_set_scales(layer, b, sc, sc)
+            else:
+                k = torch.randn((n, hkv, D), generator=g, device="cuda:0").half()
+                v = torch.randn((n, hkv, D), generator=g, device="cuda:0").half()
+            at.kv_append(layer, b, 0, k, v)
+    q = torch.randn((B, hq, D), device="cuda:0").half()
+    out = torch.empty_like(q)
+    clens = A._i32_array(lens)
+
+    def step(i):
+        at.decode(i % rotation, clens, q, out, num_splits=splits, batch=B)
+
+    sec = time_steps(torch, step, steps, warmup)
+    kms = kernel_ms(torch, at, step, min(steps, 30), warmup + steps)
+    esz = 1 if kv == A.I8 else 2
+    nbytes = sum(lens) * hkv * D * 2 * esz + 2 * B * hq * D * 2 + (B * 2 * hkv * D * 4 if kv == A.I8 else 0)
+    at.close()
+    return {"workload": name, "ms_per_step": sec * 1e3, "kernel_ms": kms, "bytes": nbytes,
+            "GBps": nbytes / sec / 1e9, "kernel_GBps": nbytes / (kms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tokens_per_s": B / sec}
+
+
+def prefill_flops(n, hq, window):
+    pairs = sum(min(i + 1, window) if window > 0 else i + 1 for i in range(n))
+    return 4 * hq * D * pairs
+
+
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024):
+    hq, hkv = 4, 1
+    windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
+    stream = torch.cuda.current_stream().cuda_stream
+    at = A.Attn(layers, hq, hkv, D, n, 1, A.BF16, A.BF16, layer_window=windows, stream=stream)
+    fill_cache(at, torch, layers, [n], hkv, torch.bfloat16, seed=0xC0FFEE + 1)
+    q = torch.randn((layers, n, hq, D), device="cuda:0").bfloat16()
+    out = torch.empty_like(q)
+
+    def step(i):
+        at.prefill(0, 0, 0, n, q, out, n_layers=layers)
+
+    sec = time_steps(torch, step, steps, warmup)
+    kms = kernel_ms(torch, at, step, min(steps, 30), 0)
+    flops = sum(prefill_flops(n, hq, w) for w in windows)
+
+    def step1(i):
+        at.prefill(5, 0, 0, n, q[5], out[5])  # one global layer
+    lat1 = time_steps(torch, step1, 50, 5)
+    at.close()
+    return {"workload": "C2: 26 layers x 1024 tokens, Hq4/Hkv1, bf16, 22 local(W=512)+4 global, one launch",
+            "ms_per_step": sec * 1e3, "kernel_ms": kms, "flops": flops, "TFLOPs": flops / sec / 1e12,
+            "kernel_TFLOPs": flops / (kms * 1e-3) / 1e12,
+            "frac_of_mfma_peak": flops / (kms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "tokens_per_s": n / sec, "single_global_layer_ms": lat1 * 1e3,
+            "dense_counted_TFLOPs": layers * 4 * hq * D * n * n / sec / 1e12}
+
+
+def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=12.0):
+    """C restatement of the reference CPU op order (fp32, OpenMP) on the same
+    30-layer decode sweep, repeated until about `budget_s` seconds are spent."""
+    from oracle import c_oracle
+    hq, hkv = 8, 2
+    rng = np.random.default_rng(0xC0FFEE + 2)
+    ks = [rng.standard_normal((ctx, hkv, D), dtype=np.float32) for _ in range(layers)]
+    vs = [rng.standard_normal((ctx, hkv, D), dtype=np.float32) for _ in range(layers)]
+    q = rng.standard_normal((layers, hq, D), dtype=np.float32)
+    res = {}
+    for threads in (4, 0):
+        c_oracle.decode_batch_ref_f32(q, ks, vs, D ** -0.5, threads=threads)  # warm
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < budget_s / 2:
+            c_oracle.decode_batch_ref_f32(q, ks, vs, D ** -0.5, threads=threads)
+            reps += 1
+        sec = (time.perf_counter() - t0) / reps
+        used = threads if threads > 0 else c_oracle.num_threads()
+        res[used] = {"sec_per_step": sec, "reps": reps}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="headline decode workload only")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference point for rocprofv3 --pmc counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from __graft_entry__ import load_package
+    A = load_package().attn
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    log(f"[bench] {A.version()} on {torch.cuda.get_device_name(0)}")
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    dec = bench_decode_c3(A, torch, args.steps, args.warmup)
+    log(f"[bench] decode C3x{dec['layers']}: {dec['sec_per_step']*1e6:.1f} us/step, kernel {dec['kernel_ms']*1e3:.1f} us")
+    value = dec["step_bytes"] / dec["sec_per_step"] / 1e9
+    achieved = dec["step_bytes"] / (dec["kernel_ms"] * 1e-3) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dec["sec_per_step"] * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "C3 x 30 layers: Gemma3n-E2B-shaped decode attention, batch 1, Hq8/Hkv2, head_dim 256, "
+                        "fp16 KV cache at 4096 context, 16 split-KV partitions + LSE merge, one multi-layer launch "
+                        "per step, rotating over 4 cache sets (1 GiB) so reads come from HBM",
+            "layers_per_step": dec["layers"], "context": 4096, "num_splits": 16,
+            "algorithmic_bytes_per_step": dec["step_bytes"],
+        },
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "decode_steps_per_s": round(dec["tokens_per_s"], 1),
+        "single_layer_latency_us": round(dec["single_layer_latency_us"], 2),
+        "roofline": {
+            "kernel": "decode_attn_kernel<f16,f16,256>",
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES,
+            "algorithmic_bytes_per_launch": dec["step_bytes"],
+            "avg_kernel_us": round(dec["kernel_ms"] * 1e3, 2),
+        },
+    }
+
+    if not args.no_extras:
+        pre = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4))
+        log(f"[bench] prefill C2: {pre['ms_per_step']:.3f} ms/step, {pre['kernel_TFLOPs']:.1f} TFLOP/s kernel")
+        result["prefill"] = {
+            "workload": pre["workload"], "value": round(pre["TFLOPs"], 2), "unit": "TFLOP/s", "dtype": "bf16",
+            "ms_per_step": round(pre["ms_per_step"], 4), "prefill_tokens_per_s": round(pre["tokens_per_s"], 1),
+            "single_global_layer_ms": round(pre["single_global_layer_ms"], 4),
+            "dense_counted_TFLOPs": round(pre["dense_counted_TFLOPs"], 2),
+            "roofline": {"kernel": "prefill_attn_kernel<bf16,256>", "bound": "mfma",
+                         "achieved": round(pre["kernel_TFLOPs"], 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(pre["frac_of_mfma_peak"], 4), "traffic": None,
+                         "algorithmic_flops_per_launch": pre["flops"], "avg_kernel_us": round(pre["kernel_ms"] * 1e3, 2)},
+        }
+        rng = np.random.default_rng(0xC0FFEE + 3)
+        lens4 = [int(x) for x in rng.integers(256, 4097, size=64)]
+        extras = []
+        for name, kv, lens, rot in (("C4: 64 seqs, L~U[256,4096], fp16, one layer", A.F16, lens4, 4),
+                                    ("C5: 32 seqs x 4096, int8 KV + fp32 scales, one layer", A.I8, [4096] * 32, 6)):
+            r = bench_decode_batch(A, torch, name, kv, lens, max(20, args.steps // 4), max(5, args.warmup // 4), rot, 16)
+            log(f"[bench] {name}: {r['ms_per_step']*1e3:.1f} us/step, kernel {r['kernel_GBps']:.0f} GB/s")
+            extras.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        result["other_decode_configs"] = extras
+
+    if not args.no_cpu:
+        cpu = cpu_baseline_c3(dec["layers"], 4096, dec["step_bytes"])
+        used = sorted(cpu)
+        ref_threads = 4 if 4 in cpu else used[0]
+        result["cpu_baseline"] = {
+            "value": round(dec["step_bytes"] / cpu[ref_threads]["sec_per_step"] / 1e9, 3),
+            "unit": "GB/s",
+            "cores": ref_threads,
+            "kind": "port",
+            "sample": f"{cpu[ref_threads]['reps']} passes of the same 30-layer decode sweep (fp32 K/V copies, about 6 s), "
+                      "C restatement of the reference CPU op order (oracle/attn_oracle.c, OpenMP); "
+                      "4 threads = the reference's CpuConfig default; bytes counted as for the GPU (fp16 sizes)",
+            "ms_per_step": round(cpu[ref_threads]["sec_per_step"] * 1e3, 3),
+        }
+        if used[-1] != ref_threads:
+            t = used[-1]
+            result["cpu_baseline_all_cores"] = {
+                "value": round(dec["step_bytes"] / cpu[t]["sec_per_step"] / 1e9, 3), "unit": "GB/s", "cores": t,
+                "kind": "port", "ms_per_step": round(cpu[t]["sec_per_step"] * 1e3, 3)}
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

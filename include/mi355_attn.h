@@ -180,8 +180,7 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
 
 /*
  * Tuning and cross-check switches (return kInvalidArgument for unknown names):
- *   "decode_waves"     2 or 4 waves per decode workgroup (default 4)
- *   "decode_pipeline"  0/1 keep the next block's loads in flight (default 1)
+ *   "decode_waves"     1, 2 or 4 waves per decode workgroup
  *   "rowwise_prefill"  0/1 run prefill row by row through the decode kernel
  *                      (the only path for fp32 and int8 caches)
  */

@@ -40,6 +40,7 @@ MI355_HD int dtype_size(int dt) { return dt == kF32 ? 4 : (dt == kI8 ? 1 : 2); }
 
 constexpr int kTokenAlign = 64;  // planes hold a multiple of 64 rows
 constexpr int kMaxGroup = 16;    // query heads per KV head handled by one MFMA column block
+constexpr int kInlineItems = 8;  // batches up to this size need no upload of their lengths
 
 MI355_HD int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -81,8 +82,11 @@ struct DecodeArgs {
   const float* scales;       // int8 cache only
   float* ws_acc;             // [items][hq][num_splits][D] partial accumulators
   float* ws_ml;              // [items][hq][num_splits][2] partial (max, sum)
-  const int32_t* kv_lens;    // [batch]
+  const int32_t* kv_lens;    // [batch] (unused when inline_items != 0)
   const int32_t* seq_ids;    // [batch] or nullptr
+  int32_t inline_items;      // != 0: batch <= kInlineItems and lens / sequence ids travel in the argument block
+  int32_t inline_lens[kInlineItems];
+  int32_t inline_seq[kInlineItems];
   const int32_t* layer_window;  // [num_layers]
   CacheGeom geom;
   int32_t hq, group;

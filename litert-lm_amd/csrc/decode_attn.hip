@@ -3,13 +3,15 @@
 // Grid: x = split-KV partition, y = KV head, z = (layer, sequence) item.
 // A workgroup of NW waves streams the K and V rows of its partition exactly
 // once. Each wave owns every NW-th block of VB tokens and, per block, issues
-// 32 wave-wide 1 KiB streaming loads (16 of K, 16 of V at head_dim 256), the
-// next block's loads before the current block's arithmetic. Scores are
+// 32 wave-wide 1 KiB streaming loads (16 of K, 16 of V at head_dim 256); the
+// K loads of the next block are issued as soon as the current scores exist and
+// the V loads right after P.V, so memory stays busy during the arithmetic. Scores are
 // S^T = K . Q^T on the matrix cores with the (at most 16) query heads of the KV
 // head in the column dimension, so each lane keeps the running max / sum of
 // one query head; the probabilities leave the first MFMA already in the
 // operand layout of the second (O^T = V^T . P^T). Waves are merged through
-// LDS, partitions through a workspace and a small log-sum-exp merge kernel.
+// LDS; partitions write (max, sum, accumulator) partials to a workspace that a
+// small second kernel merges by log-sum-exp.
 //
 // Replaces the decode-time attention that the reference reaches through
 // compiled_model_.Run("decode", ...)
@@ -46,111 +48,131 @@ struct IoT<kF16> { using type = _Float16; };
 template <>
 struct IoT<kBF16> { using type = __bf16; };
 
-// K and V bytes of one block of VB tokens as they sit in a wave's registers.
-template <int D>
-struct BlockRegs {
-  u4 k[D / 16];
-  u4 v[D / 16];
-};
+// A block of VB tokens is 64*D bytes in both planes, laid out so that load i
+// of a wave is bytes [i*1024, (i+1)*1024) of the block. Buffer loads keep the
+// plane base and the block offset in scalar registers (one VGPR of address per
+// lane for all 32 loads) and are bounds-checked against the plane size.
+constexpr int kStreamingLoad = 2;  // "nt": the rows are read once per call
 
-template <int D>
-__device__ __forceinline__ void load_block(BlockRegs<D>& r, const uint8_t* kblock, const uint8_t* vblock,
-                                           int lane) {
-  // A block is 64*D bytes in both planes, laid out so that load i of a wave is
-  // bytes [i*1024, (i+1)*1024) of the block.
-#pragma unroll
-  for (int i = 0; i < D / 16; ++i) r.k[i] = load_stream16(kblock + i * 1024 + lane * 16);
-#pragma unroll
-  for (int i = 0; i < D / 16; ++i) r.v[i] = load_stream16(vblock + i * 1024 + lane * 16);
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_resource(const uint8_t* plane, int64_t plane_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(plane), 0, (int)plane_bytes, 0x00020000);
 }
 
-// Q^T as the B operand: lane (n = lane%16, g = lane/16) holds, for chunk step
-// jj, the elements of head n that pair with K chunk 4*jj + g. Heads n >= group
-// are zero columns.
+template <int D>
+__device__ __forceinline__ void load_plane_block(u4 (&r)[D / 16], __amdgpu_buffer_rsrc_t rsrc, int block_off,
+                                                 int lane_off) {
+#pragma unroll
+  for (int i = 0; i < D / 16; ++i)
+    r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + (i & 3) * 1024, block_off + (i >> 2) * 4096,
+                                                 kStreamingLoad);
+}
+
+// Q^T as the B operand, staged once per workgroup in LDS as [step][lane] 16-byte
+// entries: entry (jj, lane) with n = lane%16, g = lane/16 holds the elements of
+// query head n that pair with K chunk 4*jj + g (for an int8 cache: with one
+// half of that chunk, pre-multiplied by the K scales). Heads n >= group are
+// zero columns. Keeping Q out of the register file leaves room for two waves
+// per SIMD next to the 128 registers of K/V data in flight.
 template <int KV, int IO, int D>
-__device__ __forceinline__ void load_q(u4 (&qreg)[KV == kF32 ? D / 16 : D / 32], const DecodeArgs& a,
-                                       int item, int kvh, int seq, int layer, int lane) {
+__device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, int item, int kvh, int seq, int layer,
+                                        int nthreads) {
   using io_t = typename IoT<IO>::type;
   constexpr int EPC = KvT<KV>::EPC;
-  const int n = lane & 15, g = lane >> 4;
-  const bool live = n < a.group;
-  const io_t* qrow = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group + (live ? n : 0)) * D;
-  if constexpr (KV == kI8) {
-    static_assert(IO == kF16, "int8 cache pairs with fp16 queries");
-    const float* ks = a.scales + a.geom.scale_offset(layer, seq, 0, kvh);
+  constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
+  for (int idx = threadIdx.x; idx < NQ * 64; idx += nthreads) {
+    const int step = idx >> 6, l = idx & 63;
+    const int n = l & 15, g = l >> 4;
+    const bool live = n < a.group;
+    const io_t* qrow =
+        reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group + (live ? n : 0)) * D;
+    u4 w;
+    if constexpr (KV == kI8) {
+      static_assert(IO == kF16, "int8 cache pairs with fp16 queries");
+      const float* ks = a.scales + a.geom.scale_offset(layer, seq, 0, kvh);
+      const int d0 = (4 * (step >> 1) + g) * EPC + 8 * (step & 1);
+      const h8 qv = *reinterpret_cast<const h8*>(qrow + d0);
+      h8 o;
 #pragma unroll
-    for (int jj = 0; jj < D / 64; ++jj) {
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int d0 = (4 * jj + g) * EPC + 8 * half;
-        h8 qv = *reinterpret_cast<const h8*>(qrow + d0);
-        h8 o;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = live ? (_Float16)((float)qv[e] * ks[d0 + e]) : (_Float16)0;
-        qreg[2 * jj + half] = bit_cast<u4>(o);
-      }
+      for (int e = 0; e < 8; ++e) o[e] = (_Float16)((float)qv[e] * ks[d0 + e]);
+      w = bit_cast<u4>(o);
+    } else {
+      w = *reinterpret_cast<const u4*>(qrow + (4 * step + g) * EPC);
     }
-  } else {
-    constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
-#pragma unroll
-    for (int jj = 0; jj < NQ; ++jj) {
-      u4 w = *reinterpret_cast<const u4*>(qrow + (4 * jj + g) * EPC);
-      qreg[jj] = live ? w : u4{0, 0, 0, 0};
-    }
+    sm_q[idx] = live ? w : u4{0, 0, 0, 0};
   }
 }
 
 // S^T tiles of one block: s[T][i] is the raw score of token 16*T + 4*g + i
-// against head n.
+// against head n. sm_q[step * 64 + qi] is this lane's Q operand of a step; each
+// is read once and used for every tile of the block.
 template <int KV, int D>
-__device__ __forceinline__ void qk_block(const BlockRegs<D>& r, const u4 (&qreg)[KV == kF32 ? D / 16 : D / 32],
+__device__ __forceinline__ void qk_block(const u4 (&kreg)[D / 16], const u4* sm_q, int qi,
                                          f4 (&s)[KvT<KV>::VB / 16]) {
   constexpr int NT = KvT<KV>::VB / 16;
   constexpr int KPT = (D / 16) / NT;  // K loads per 16-token tile
 #pragma unroll
-  for (int T = 0; T < NT; ++T) {
-    f4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int T = 0; T < NT; ++T) s[T] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < KPT; ++j) {
-      const u4 kw = r.k[T * KPT + j];
-      if constexpr (KV == kF16) {
-        acc = mfma16_f16(bit_cast<h8>(kw), bit_cast<h8>(qreg[j]), acc);
-      } else if constexpr (KV == kBF16) {
-        acc = mfma16_bf16(bit_cast<b8>(kw), bit_cast<b8>(qreg[j]), acc);
-      } else if constexpr (KV == kF32) {
-        const f4 kf = bit_cast<f4>(kw), qf = bit_cast<f4>(qreg[j]);
+  for (int j = 0; j < KPT; ++j) {
+    if constexpr (KV == kF16) {
+      const h8 qv = bit_cast<h8>(sm_q[j * 64 + qi]);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc = mfma16_f32(kf[e], qf[e], acc);
-      } else {
+      for (int T = 0; T < NT; ++T) s[T] = mfma16_f16(bit_cast<h8>(kreg[T * KPT + j]), qv, s[T]);
+    } else if constexpr (KV == kBF16) {
+      const b8 qv = bit_cast<b8>(sm_q[j * 64 + qi]);
+#pragma unroll
+      for (int T = 0; T < NT; ++T) s[T] = mfma16_bf16(bit_cast<b8>(kreg[T * KPT + j]), qv, s[T]);
+    } else if constexpr (KV == kF32) {
+      const f4 qf = bit_cast<f4>(sm_q[j * 64 + qi]);
+#pragma unroll
+      for (int T = 0; T < NT; ++T) {
+        const f4 kf = bit_cast<f4>(kreg[T * KPT + j]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[T] = mfma16_f32(kf[e], qf[e], s[T]);
+      }
+    } else {
+      const h8 q0 = bit_cast<h8>(sm_q[(2 * j) * 64 + qi]), q1 = bit_cast<h8>(sm_q[(2 * j + 1) * 64 + qi]);
+#pragma unroll
+      for (int T = 0; T < NT; ++T) {
         h8 lo, hi;
-        cvt_i8x16_to_h8x2(kw, lo, hi);
-        acc = mfma16_f16(lo, bit_cast<h8>(qreg[2 * j]), acc);
-        acc = mfma16_f16(hi, bit_cast<h8>(qreg[2 * j + 1]), acc);
+        cvt_i8x16_to_h8x2(kreg[T * KPT + j], lo, hi);
+        s[T] = mfma16_f16(lo, q0, s[T]);
+        s[T] = mfma16_f16(hi, q1, s[T]);
       }
     }
-    s[T] = acc;
   }
 }
 
 // O^T += V^T . P^T for one block; p[T][i] pairs with token 16*T + 4*g + i.
 template <int KV, int D>
-__device__ __forceinline__ void pv_block(const BlockRegs<D>& r, const f4 (&p)[KvT<KV>::VB / 16], f4 (&acc)[D / 16]) {
+__device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)[KvT<KV>::VB / 16], f4 (&acc)[D / 16]) {
   if constexpr (KV == kF16) {
     h8 pp;
 #pragma unroll
     for (int e = 0; e < 4; ++e) { pp[e] = (_Float16)p[0][e]; pp[4 + e] = (_Float16)p[1][e]; }
 #pragma unroll
-    for (int db = 0; db < D / 16; ++db) acc[db] = mfma16_f16(bit_cast<h8>(r.v[db]), pp, acc[db]);
+    for (int db = 0; db < D / 16; ++db) acc[db] = mfma16_f16(bit_cast<h8>(vreg[db]), pp, acc[db]);
   } else if constexpr (KV == kBF16) {
-    b8 pp;
+    // bf16 keeps 8 significant bits: P is fed as hi + lo parts (two MFMAs, the
+    // matrix cores are idle most of the time here) so that the probabilities
+    // enter P.V with ~16 bits instead of adding ~1e-3 of relative error.
+    b8 hi, lo;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { pp[e] = (__bf16)p[0][e]; pp[4 + e] = (__bf16)p[1][e]; }
+    for (int e = 0; e < 4; ++e) {
+      hi[e] = (__bf16)p[0][e];
+      hi[4 + e] = (__bf16)p[1][e];
+      lo[e] = (__bf16)(p[0][e] - (float)hi[e]);
+      lo[4 + e] = (__bf16)(p[1][e] - (float)hi[4 + e]);
+    }
 #pragma unroll
-    for (int db = 0; db < D / 16; ++db) acc[db] = mfma16_bf16(bit_cast<b8>(r.v[db]), pp, acc[db]);
+    for (int db = 0; db < D / 16; ++db) {
+      acc[db] = mfma16_bf16(bit_cast<b8>(vreg[db]), hi, acc[db]);
+      acc[db] = mfma16_bf16(bit_cast<b8>(vreg[db]), lo, acc[db]);
+    }
   } else if constexpr (KV == kF32) {
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {
-      const f4 vf = bit_cast<f4>(r.v[db]);
+      const f4 vf = bit_cast<f4>(vreg[db]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[db] = mfma16_f32(vf[e], p[0][e], acc[db]);
     }
@@ -164,26 +186,63 @@ __device__ __forceinline__ void pv_block(const BlockRegs<D>& r, const f4 (&p)[Kv
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {
       h8 lo, hi;
-      cvt_i8x16_to_h8x2(r.v[db], lo, hi);
+      cvt_i8x16_to_h8x2(vreg[db], lo, hi);
       acc[db] = mfma16_f16(lo, p01, acc[db]);
       acc[db] = mfma16_f16(hi, p23, acc[db]);
     }
   }
 }
 
-template <int KV, int IO, int D, int NW, bool PIPE>
-__global__ void __launch_bounds__(NW * 64) decode_attn_kernel(const DecodeArgs a) {
+// Log-sum-exp merge of the split-KV partials: grid (query head, item), one
+// thread per channel. A separate launch because partials written by workgroups
+// on other XCDs are only guaranteed visible across a kernel boundary; an
+// in-kernel "last arrival merges" needs an L2 write-back and invalidate per
+// workgroup, which measured several times slower than this launch.
+template <int KV, int IO, int D>
+__global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
+  using io_t = typename IoT<IO>::type;
+  const int head = blockIdx.x, item = blockIdx.y, d = threadIdx.x;
+  const int li = item / a.batch, b = item - li * a.batch;
+  const int layer = a.layer_begin + li;
+  const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
+  const int window = a.layer_window[layer];
+  int vlo, start;
+  decode_visible_range(kv_len, window, &vlo, &start);
+  const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
+  int nparts = (kv_len - start + per - 1) / per;
+  nparts = nparts < a.num_splits ? nparts : a.num_splits;
+  const int64_t slot0 = ((int64_t)item * a.hq + head) * a.num_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < nparts; ++s) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
+  const float m_use = (M == -INFINITY) ? 0.f : M;
+  float A = 0.f, L = 0.f;
+  for (int s = 0; s < nparts; ++s) {
+    const float wgt = fast_exp2(a.ws_ml[(slot0 + s) * 2] - m_use);
+    A += wgt * a.ws_acc[(slot0 + s) * D + d];
+    L += wgt * a.ws_ml[(slot0 + s) * 2 + 1];
+  }
+  float o = L > 0.f ? A / L : 0.f;
+  if constexpr (KV == kI8) {
+    const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
+    o *= a.scales[a.geom.scale_offset(layer, seq, 1, head / a.group) + d];
+  }
+  reinterpret_cast<io_t*>(a.out)[((int64_t)item * a.hq + head) * D + d] = (io_t)o;
+}
+
+template <int KV, int IO, int D, int NW>
+__global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
   constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   extern __shared__ float smem[];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: block addresses stay scalar
   const int n = lane & 15, g = lane >> 4;
   const int split = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z;
   const int li = item / a.batch, b = item - li * a.batch;
   const int layer = a.layer_begin + li;
-  const int seq = a.seq_ids ? a.seq_ids[b] : b;
-  const int kv_len = a.kv_lens[b];
+  const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
+  const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
   const int window = a.layer_window[layer];
   int vlo, start;
   decode_visible_range(kv_len, window, &vlo, &start);
@@ -193,38 +252,69 @@ __global__ void __launch_bounds__(NW * 64) decode_attn_kernel(const DecodeArgs a
   if (p_lo >= p_hi) return;  // empty partition: uniform over the workgroup
 
   const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, seq, kvh, 0);
-  const uint8_t* vplane = kplane + a.geom.plane_bytes;
-  constexpr int64_t kBlockBytes = 64 * D;
+  const __amdgpu_buffer_rsrc_t krsrc = plane_resource(kplane, a.geom.plane_bytes);
+  const __amdgpu_buffer_rsrc_t vrsrc = plane_resource(kplane + a.geom.plane_bytes, a.geom.plane_bytes);
+  constexpr int kBlockBytes = 64 * D;
+  const int blk_end = (p_hi + VB - 1) / VB;
+  const int lane_off = lane * 16;
 
-  u4 qreg[NQ];
-  load_q<KV, IO, D>(qreg, a, item, kvh, seq, layer, lane);
+  // Rolling prefetch: the K registers are refilled with the next block as soon
+  // as the QK^T product has consumed them, the V registers right after P.V, so
+  // 16 to 32 KiB per wave are in flight while it computes.
+  u4 kreg[NL], vreg[NL];
+  int blk = __builtin_amdgcn_readfirstlane(p_lo / VB + wave);
+  if (blk < blk_end) {
+    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
+    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
+  }
+  u4* sm_q = reinterpret_cast<u4*>(smem);
+  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, NW * 64);
+  __syncthreads();
 
   float m_run = -INFINITY, l_run = 0.f;
   f4 acc[NL];
 #pragma unroll
   for (int i = 0; i < NL; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
-
   const float sc = a.scale, softcap = a.softcap;
-  const int blk_end = (p_hi + VB - 1) / VB;
 
-  auto process = [&](const BlockRegs<D>& r, int blk) {
+  while (blk < blk_end) {
+    // The index is made opaque so the Q reads stay inside the loop: hoisted
+    // they would occupy 32 to 64 registers for the whole kernel.
+    int qi = lane;
+    asm volatile("" : "+v"(qi));
     f4 s[NT];
-    qk_block<KV, D>(r, qreg, s);
-    const int tok0 = blk * VB + 4 * g;
+    qk_block<KV, D>(kreg, sm_q, qi, s);
+    const int nxt = blk + NW;
+    if (nxt < blk_end) load_plane_block<D>(kreg, krsrc, nxt * kBlockBytes, lane_off);
+
+    // scores in the exp2 domain; soft-capping and the range mask are uniform
+    // branches taken only by the layers / boundary blocks that need them
+    if (softcap > 0.f) {
+      const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
+#pragma unroll
+      for (int T = 0; T < NT; ++T)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[T][i] = cap2 * fast_tanh(s[T][i] * inv_cap);
+    } else {
+      const float sc2 = sc * kLog2e;
+#pragma unroll
+      for (int T = 0; T < NT; ++T) s[T] *= sc2;
+    }
+    if (blk * VB < vlo || (blk + 1) * VB > p_hi) {
+      const int tok0 = blk * VB + 4 * g;
+#pragma unroll
+      for (int T = 0; T < NT; ++T)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = tok0 + 16 * T + i;
+          s[T][i] = (tok >= vlo && tok < p_hi) ? s[T][i] : -INFINITY;
+        }
+    }
     float bm = -INFINITY;
 #pragma unroll
-    for (int T = 0; T < NT; ++T) {
+    for (int T = 0; T < NT; ++T)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = tok0 + 16 * T + i;
-        float x = s[T][i] * sc;
-        if (softcap > 0.f) x = softcap * tanhf(x / softcap);
-        x *= kLog2e;
-        x = (tok >= vlo && tok < p_hi) ? x : -INFINITY;
-        s[T][i] = x;
-        bm = fmaxf(bm, x);
-      }
-    }
+      for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[T][i]);
     bm = wave_xor_max(bm, 16);
     bm = wave_xor_max(bm, 32);
     const float m_new = fmaxf(m_run, bm);
@@ -241,33 +331,12 @@ __global__ void __launch_bounds__(NW * 64) decode_attn_kernel(const DecodeArgs a
       }
     }
     l_run = l_run * alpha + lsum;
+    m_run = m_new;
 #pragma unroll
     for (int i = 0; i < NL; ++i) acc[i] *= alpha;
-    pv_block<KV, D>(r, s, acc);
-    m_run = m_new;
-  };
-
-  int blk = p_lo / VB + wave;
-  if constexpr (PIPE) {
-    BlockRegs<D> ra, rb;
-    if (blk < blk_end) load_block<D>(ra, kplane + blk * kBlockBytes, vplane + blk * kBlockBytes, lane);
-    while (blk < blk_end) {
-      if (blk + NW < blk_end)
-        load_block<D>(rb, kplane + (blk + NW) * kBlockBytes, vplane + (blk + NW) * kBlockBytes, lane);
-      process(ra, blk);
-      blk += NW;
-      if (blk >= blk_end) break;
-      if (blk + NW < blk_end)
-        load_block<D>(ra, kplane + (blk + NW) * kBlockBytes, vplane + (blk + NW) * kBlockBytes, lane);
-      process(rb, blk);
-      blk += NW;
-    }
-  } else {
-    for (; blk < blk_end; blk += NW) {
-      BlockRegs<D> r;
-      load_block<D>(r, kplane + blk * kBlockBytes, vplane + blk * kBlockBytes, lane);
-      process(r, blk);
-    }
+    pv_block<KV, D>(vreg, s, acc);
+    if (nxt < blk_end) load_plane_block<D>(vreg, vrsrc, nxt * kBlockBytes, lane_off);
+    blk = nxt;
   }
 
   // The four lanes (g = 0..3) of a head each summed their own tokens.
@@ -276,7 +345,7 @@ __global__ void __launch_bounds__(NW * 64) decode_attn_kernel(const DecodeArgs a
 
   // Merge the waves through LDS: [NW][group][D] accumulators, then max, sum.
   const int G = a.group;
-  float* sm_acc = smem;
+  float* sm_acc = smem + NQ * 64 * 4;  // behind the staged Q
   float* sm_m = sm_acc + NW * G * D;
   float* sm_l = sm_m + NW * G;
   if (n < G) {
@@ -320,64 +389,26 @@ __global__ void __launch_bounds__(NW * 64) decode_attn_kernel(const DecodeArgs a
   }
 }
 
-// Log-sum-exp merge of the split-KV partials: grid (query head, item), one
-// thread per channel.
-template <int KV, int IO, int D>
-__global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
-  using io_t = typename IoT<IO>::type;
-  const int head = blockIdx.x, item = blockIdx.y, d = threadIdx.x;
-  const int li = item / a.batch, b = item - li * a.batch;
-  const int layer = a.layer_begin + li;
-  const int kv_len = a.kv_lens[b];
-  const int window = a.layer_window[layer];
-  int vlo, start;
-  decode_visible_range(kv_len, window, &vlo, &start);
-  const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
-  int nparts = (kv_len - start + per - 1) / per;
-  nparts = nparts < a.num_splits ? nparts : a.num_splits;
-  const int64_t slot0 = ((int64_t)item * a.hq + head) * a.num_splits;
-  float M = -INFINITY;
-  for (int s = 0; s < nparts; ++s) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
-  const float m_use = (M == -INFINITY) ? 0.f : M;
-  float A = 0.f, L = 0.f;
-  for (int s = 0; s < nparts; ++s) {
-    const float wgt = fast_exp2(a.ws_ml[(slot0 + s) * 2] - m_use);
-    A += wgt * a.ws_acc[(slot0 + s) * D + d];
-    L += wgt * a.ws_ml[(slot0 + s) * 2 + 1];
-  }
-  float o = L > 0.f ? A / L : 0.f;
-  if constexpr (KV == kI8) {
-    const int seq = a.seq_ids ? a.seq_ids[b] : b;
-    o *= a.scales[a.geom.scale_offset(layer, seq, 1, head / a.group) + d];
-  }
-  reinterpret_cast<io_t*>(a.out)[((int64_t)item * a.hq + head) * D + d] = (io_t)o;
-}
-
-template <int KV, int IO, int D, int NW, bool PIPE>
+template <int KV, int IO, int D, int NW>
 hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int items = a.n_layers * a.batch;
   const dim3 grid(a.num_splits, a.geom.hkv, items);
-  const size_t lds = (size_t)NW * a.group * (D + 2) * sizeof(float);
+  constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
+  const size_t lds = (size_t)NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
   if (ev0) (void)hipEventRecord(ev0, stream);
-  hipLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, PIPE>), grid, dim3(NW * 64), lds, stream, a);
+  hipLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW>), grid, dim3(NW * 64), lds, stream, a);
   if (ev1) (void)hipEventRecord(ev1, stream);
   hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return err;
-  if (a.num_splits > 1) {
-    hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D>), dim3(a.hq, items), dim3(D), 0, stream, a);
-    err = hipGetLastError();
-  }
-  return err;
+  if (err != hipSuccess || a.num_splits == 1) return err;
+  hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D>), dim3(a.hq, items), dim3(D), 0, stream, a);
+  return hipGetLastError();
 }
 
 template <int KV, int IO, int D>
 hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t s, hipEvent_t e0, hipEvent_t e1) {
-  if (t.waves == 2) {
-    return t.pipeline ? launch_variant<KV, IO, D, 2, true>(a, s, e0, e1)
-                      : launch_variant<KV, IO, D, 2, false>(a, s, e0, e1);
-  }
-  return t.pipeline ? launch_variant<KV, IO, D, 4, true>(a, s, e0, e1)
-                    : launch_variant<KV, IO, D, 4, false>(a, s, e0, e1);
+  if (t.waves == 1) return launch_variant<KV, IO, D, 1>(a, s, e0, e1);
+  if (t.waves == 2) return launch_variant<KV, IO, D, 2>(a, s, e0, e1);
+  return launch_variant<KV, IO, D, 4>(a, s, e0, e1);
 }
 
 }  // namespace

@@ -10,8 +10,7 @@
 namespace mi355 {
 
 struct DecodeTuning {
-  int waves = 4;         // waves per workgroup (2 or 4)
-  bool pipeline = true;  // keep the next block's loads in flight during arithmetic
+  int waves = 2;  // waves per workgroup: 1, 2 or 4
 };
 
 bool decode_supported(int kv_dtype, int io_dtype, int head_dim);

@@ -71,6 +71,13 @@ __device__ __forceinline__ void cvt_i8x16_to_h8x2(u4 w, h8& lo, h8& hi) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// tanh(y) = sign(y) * (1 - t) / (1 + t), t = exp(-2|y|): no overflow, no branch.
+__device__ __forceinline__ float fast_tanh(float y) {
+  const float t = __builtin_amdgcn_exp2f(-2.8853900817779268f * fabsf(y));
+  const float r = (1.f - t) * __builtin_amdgcn_rcpf(1.f + t);
+  return copysignf(r, y);
+}
+
 __device__ __forceinline__ float wave_xor_max(float v, int mask) { return fmaxf(v, __shfl_xor(v, mask, 64)); }
 __device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
 

@@ -75,6 +75,7 @@ struct mi355_attn {
   float* ws_acc = nullptr;
   float* ws_ml = nullptr;
   size_t ws_slots = 0;
+
   // ring of (kv_lens, seq_ids) uploads
   int32_t* h_ring = nullptr;
   int32_t* d_ring = nullptr;
@@ -241,7 +242,15 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   void* dout = nullptr;
   if (int rc = stage_in(h, 0, q, io_bytes, &dq, error_msg)) return rc;
   if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
-  if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, error_msg)) return rc;
+  if (batch <= kInlineItems) {
+    a.inline_items = 1;
+    for (int b = 0; b < batch; ++b) {
+      a.inline_lens[b] = kv_lens[b];
+      a.inline_seq[b] = seq_ids ? seq_ids[b] : b;
+    }
+  } else if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, error_msg)) {
+    return rc;
+  }
   a.q = dq;
   a.out = dout;
   a.layer_begin = layer_begin;
@@ -396,8 +405,6 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
   h->geom.esize = dtype_size(c->kv_dtype);
   h->geom.plane_bytes = (int64_t)h->geom.cap * c->head_dim * h->geom.esize;
   h->cache_bytes = (uint64_t)h->geom.plane_bytes * 2 * c->num_kv_heads * c->max_seqs * c->num_layers;
-  if (const char* e = getenv("MI355_ATTN_DECODE_WAVES")) h->tuning.waves = atoi(e) == 2 ? 2 : 4;
-  if (const char* e = getenv("MI355_ATTN_DECODE_PIPELINE")) h->tuning.pipeline = atoi(e) != 0;
 
   auto bail = [&](int code, const char* what, hipError_t e) {
     int rc = fail(error_msg, code, "%s: %s", what, hipGetErrorString(e));
@@ -608,10 +615,8 @@ float mi355_attn_last_kernel_ms(mi355_attn* h) {
 int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   if (!h || !name) return MI355_ATTN_INVALID_ARGUMENT;
   if (!strcmp(name, "decode_waves")) {
-    if (value != 2 && value != 4) return MI355_ATTN_INVALID_ARGUMENT;
+    if (value != 1 && value != 2 && value != 4) return MI355_ATTN_INVALID_ARGUMENT;
     h->tuning.waves = value;
-  } else if (!strcmp(name, "decode_pipeline")) {
-    h->tuning.pipeline = value != 0;
   } else if (!strcmp(name, "rowwise_prefill")) {
     h->rowwise_prefill = value != 0;
   } else {

@@ -190,14 +190,34 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) 
     }
 
     // ---- O^T += V^T . P^T
-    vec8 p0, p1;
+    const uint8_t* vb_base = sm_v + (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
+    if constexpr (DT == kBF16) {
+      // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
+      // them, otherwise P.V alone carries ~1e-3 of relative error.
+      vec8 p0, p1, q0, q1;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      p0[e] = (elem_t)s[e];
-      p1[e] = (elem_t)s[8 + e];
-    }
-    {
-      const uint8_t* vb_base = sm_v + (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
+      for (int e = 0; e < 8; ++e) {
+        p0[e] = (elem_t)s[e];
+        p1[e] = (elem_t)s[8 + e];
+        q0[e] = (elem_t)(s[e] - (float)p0[e]);
+        q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
+      }
+#pragma unroll
+      for (int dp = 0; dp < NDP; ++dp) {
+        const vec8 v0 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048);
+        const vec8 v1 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048 + 512);
+        acc[dp] = E::mfma(v0, p0, acc[dp]);
+        acc[dp] = E::mfma(v1, p1, acc[dp]);
+        acc[dp] = E::mfma(v0, q0, acc[dp]);
+        acc[dp] = E::mfma(v1, q1, acc[dp]);
+      }
+    } else {
+      vec8 p0, p1;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p0[e] = (elem_t)s[e];
+        p1[e] = (elem_t)s[8 + e];
+      }
 #pragma unroll
       for (int dp = 0; dp < NDP; ++dp) {
         const vec8 v0 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048);

@@ -130,14 +130,12 @@ def test_decode_c1_fp32_all_variants():
     k, v = gen(seed + 100, 1024, 1, D), gen(seed + 200, 1024, 1, D)
     with make(1, 4, 1, 1024, 1, A.F32) as at:
         kr, vr = fill_seq(at, A.F32, 0, 0, k, v)
-        for waves in (4, 2):
-            for pipe in (0, 1):
-                at.set_option("decode_waves", waves)
-                at.set_option("decode_pipeline", pipe)
-                for ns in (1, 2, 16, 0):
-                    err, _ = run_decode(at, A.F32, q, [(kr, vr)], [1024], num_splits=ns)
-                    say(f"C1 fp32 waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
-                    assert err < TOL[A.F32]
+        for waves in (4, 2, 1):
+            at.set_option("decode_waves", waves)
+            for ns in (1, 2, 16, 0):
+                err, _ = run_decode(at, A.F32, q, [(kr, vr)], [1024], num_splits=ns)
+                say(f"C1 fp32 waves={waves} splits={ns}: rel_err={err:.3e}")
+                assert err < TOL[A.F32]
 
 
 @pytest.mark.parametrize("kv", [A.F16, A.BF16])
@@ -147,14 +145,12 @@ def test_decode_c3_split16(kv):
     k, v = gen(seed + 100, 4096, 2, D), gen(seed + 200, 4096, 2, D)
     with make(1, 8, 2, 4096, 1, kv) as at:
         kr, vr = fill_seq(at, kv, 0, 0, k, v)
-        for waves in (4, 2):
-            for pipe in (0, 1):
-                at.set_option("decode_waves", waves)
-                at.set_option("decode_pipeline", pipe)
-                for ns in (16, 1, 5):
-                    err, _ = run_decode(at, kv, q, [(kr, vr)], [4096], num_splits=ns)
-                    say(f"C3 kv={kv} waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
-                    assert err < TOL[kv]
+        for waves in (4, 2, 1):
+            at.set_option("decode_waves", waves)
+            for ns in (16, 1, 5):
+                err, _ = run_decode(at, kv, q, [(kr, vr)], [4096], num_splits=ns)
+                say(f"C3 kv={kv} waves={waves} splits={ns}: rel_err={err:.3e}")
+                assert err < TOL[kv]
 
 
 @pytest.mark.parametrize("kv", [A.F32, A.F16, A.BF16])
@@ -208,14 +204,12 @@ def test_decode_int8_kv():
             at.kv_set_scales(0, b, torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
             kvs.append((orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs)))
         q = gen(9, len(lens), 8, D)
-        for waves in (4, 2):
-            for pipe in (0, 1):
-                at.set_option("decode_waves", waves)
-                at.set_option("decode_pipeline", pipe)
-                for ns in (1, 16):
-                    err, _ = run_decode(at, A.I8, q, kvs, lens, num_splits=ns)
-                    say(f"int8 waves={waves} pipe={pipe} splits={ns}: rel_err={err:.3e}")
-                    assert err < TOL[A.I8]
+        for waves in (4, 2, 1):
+            at.set_option("decode_waves", waves)
+            for ns in (1, 16):
+                err, _ = run_decode(at, A.I8, q, kvs, lens, num_splits=ns)
+                say(f"int8 waves={waves} splits={ns}: rel_err={err:.3e}")
+                assert err < TOL[A.I8]
 
 
 def test_decode_softcap_and_scale():
