@@ -41,6 +41,8 @@ MI355_HD int dtype_size(int dt) { return dt == kF32 ? 4 : (dt == kI8 ? 1 : 2); }
 constexpr int kTokenAlign = 64;  // planes hold a multiple of 64 rows
 constexpr int kMaxGroup = 16;    // query heads per KV head handled by one MFMA column block
 constexpr int kInlineItems = 8;  // batches up to this size need no upload of their lengths
+constexpr int kMaxDecodeSplits = 256;
+constexpr int kInlineLayers = 64;  // calls over up to this many layers carry their windows in the argument block
 
 MI355_HD int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -87,7 +89,8 @@ struct DecodeArgs {
   int32_t inline_items;      // != 0: batch <= kInlineItems and lens / sequence ids travel in the argument block
   int32_t inline_lens[kInlineItems];
   int32_t inline_seq[kInlineItems];
-  const int32_t* layer_window;  // [num_layers]
+  const int32_t* layer_window;  // [num_layers] (read only when n_layers > kInlineLayers)
+  int32_t inline_window[kInlineLayers];  // windows of layers layer_begin .. layer_begin + n_layers - 1
   CacheGeom geom;
   int32_t hq, group;
   int32_t layer_begin, n_layers, batch;

@@ -21,6 +21,8 @@
 
 #include "attn_params.h"
 #include "kernels.h"
+#include <hip/hip_ext.h>
+
 #include "mfma_util.h"
 
 namespace mi355 {
@@ -67,24 +69,24 @@ __device__ __forceinline__ void load_plane_block(u4 (&r)[D / 16], __amdgpu_buffe
                                                  kStreamingLoad);
 }
 
-// Q^T as the B operand, staged once per workgroup in LDS as [step][lane] 16-byte
-// entries: entry (jj, lane) with n = lane%16, g = lane/16 holds the elements of
-// query head n that pair with K chunk 4*jj + g (for an int8 cache: with one
-// half of that chunk, pre-multiplied by the K scales). Heads n >= group are
-// zero columns. Keeping Q out of the register file leaves room for two waves
-// per SIMD next to the 128 registers of K/V data in flight.
+// Q^T as the B operand, kept by every wave in its own LDS slice as [step][lane]
+// 16-byte entries: entry (jj, lane) with n = lane%16, g = lane/16 holds the
+// elements of query head n that pair with K chunk 4*jj + g (for an int8 cache:
+// with one half of that chunk, pre-multiplied by the K scales). Heads
+// n >= group are zero columns. A lane only ever reads the entries it wrote
+// itself, so no barrier is needed; keeping Q out of the register file leaves
+// room for two waves per SIMD next to the 128 registers of K/V data in flight.
 template <int KV, int IO, int D>
 __device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, int item, int kvh, int seq, int layer,
-                                        int nthreads) {
+                                        int lane) {
   using io_t = typename IoT<IO>::type;
   constexpr int EPC = KvT<KV>::EPC;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
-  for (int idx = threadIdx.x; idx < NQ * 64; idx += nthreads) {
-    const int step = idx >> 6, l = idx & 63;
-    const int n = l & 15, g = l >> 4;
-    const bool live = n < a.group;
-    const io_t* qrow =
-        reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group + (live ? n : 0)) * D;
+  const int n = lane & 15, g = lane >> 4;
+  const bool live = n < a.group;
+  const io_t* qrow = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group + (live ? n : 0)) * D;
+#pragma unroll
+  for (int step = 0; step < NQ; ++step) {
     u4 w;
     if constexpr (KV == kI8) {
       static_assert(IO == kF16, "int8 cache pairs with fp16 queries");
@@ -98,7 +100,7 @@ __device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, int item,
     } else {
       w = *reinterpret_cast<const u4*>(qrow + (4 * step + g) * EPC);
     }
-    sm_q[idx] = live ? w : u4{0, 0, 0, 0};
+    sm_q[step * 64 + lane] = live ? w : u4{0, 0, 0, 0};
   }
 }
 
@@ -201,25 +203,46 @@ __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)
 template <int KV, int IO, int D>
 __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
   using io_t = typename IoT<IO>::type;
+  __shared__ float sm_m[kMaxDecodeSplits], sm_l[kMaxDecodeSplits];
   const int head = blockIdx.x, item = blockIdx.y, d = threadIdx.x;
   const int li = item / a.batch, b = item - li * a.batch;
   const int layer = a.layer_begin + li;
   const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
-  const int window = a.layer_window[layer];
+  const int window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
   int vlo, start;
   decode_visible_range(kv_len, window, &vlo, &start);
   const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
   int nparts = (kv_len - start + per - 1) / per;
   nparts = nparts < a.num_splits ? nparts : a.num_splits;
   const int64_t slot0 = ((int64_t)item * a.hq + head) * a.num_splits;
+  // one round trip for all (max, sum) pairs, then the weights come from LDS
+  for (int s = d; s < nparts; s += D) {
+    const float2 ml = *reinterpret_cast<const float2*>(a.ws_ml + (slot0 + s) * 2);
+    sm_m[s] = ml.x;
+    sm_l[s] = ml.y;
+  }
+  __syncthreads();
   float M = -INFINITY;
-  for (int s = 0; s < nparts; ++s) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
+  for (int s = 0; s < nparts; ++s) M = fmaxf(M, sm_m[s]);
   const float m_use = (M == -INFINITY) ? 0.f : M;
   float A = 0.f, L = 0.f;
-  for (int s = 0; s < nparts; ++s) {
-    const float wgt = fast_exp2(a.ws_ml[(slot0 + s) * 2] - m_use);
-    A += wgt * a.ws_acc[(slot0 + s) * D + d];
-    L += wgt * a.ws_ml[(slot0 + s) * 2 + 1];
+  const float* accp = a.ws_acc + slot0 * D + d;
+  int s = 0;
+  for (; s + 8 <= nparts; s += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = accp[(int64_t)(s + u) * D];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float wgt = fast_exp2(sm_m[s + u] - m_use);
+      A += wgt * v[u];
+      L += wgt * sm_l[s + u];
+    }
+  }
+  for (; s < nparts; ++s) {
+    const float wgt = fast_exp2(sm_m[s] - m_use);
+    A += wgt * accp[(int64_t)s * D];
+    L += wgt * sm_l[s];
   }
   float o = L > 0.f ? A / L : 0.f;
   if constexpr (KV == kI8) {
@@ -243,7 +266,7 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   const int layer = a.layer_begin + li;
   const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
   const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
-  const int window = a.layer_window[layer];
+  const int window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
   int vlo, start;
   decode_visible_range(kv_len, window, &vlo, &start);
   const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
@@ -267,9 +290,8 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
     load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
     load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
   }
-  u4* sm_q = reinterpret_cast<u4*>(smem);
-  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, NW * 64);
-  __syncthreads();
+  u4* sm_q = reinterpret_cast<u4*>(smem) + wave * (NQ * 64);
+  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, lane);
 
   float m_run = -INFINITY, l_run = 0.f;
   f4 acc[NL];
@@ -345,7 +367,7 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
 
   // Merge the waves through LDS: [NW][group][D] accumulators, then max, sum.
   const int G = a.group;
-  float* sm_acc = smem + NQ * 64 * 4;  // behind the staged Q
+  float* sm_acc = smem + NW * NQ * 64 * 4;  // behind the waves' Q slices
   float* sm_m = sm_acc + NW * G * D;
   float* sm_l = sm_m + NW * G;
   if (n < G) {
@@ -394,10 +416,10 @@ hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev
   const int items = a.n_layers * a.batch;
   const dim3 grid(a.num_splits, a.geom.hkv, items);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
-  const size_t lds = (size_t)NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
-  if (ev0) (void)hipEventRecord(ev0, stream);
-  hipLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW>), grid, dim3(NW * 64), lds, stream, a);
-  if (ev1) (void)hipEventRecord(ev1, stream);
+  const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
+  // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
+  // begin and end timestamps, not the host-side launch latency around it.
+  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || a.num_splits == 1) return err;
   hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D>), dim3(a.hq, items), dim3(D), 0, stream, a);

@@ -23,7 +23,7 @@ using namespace mi355;
 namespace {
 
 constexpr int kRingSlots = 64;
-constexpr int kMaxSplits = 256;
+constexpr int kMaxSplits = kMaxDecodeSplits;
 
 int fail(char** error_msg, int code, const char* fmt, ...) {
   if (error_msg) {
@@ -196,6 +196,11 @@ void fill_decode_common(const mi355_attn* h, DecodeArgs* a) {
   a->softcap = h->cfg.softcap;
 }
 
+void fill_inline_windows(const mi355_attn* h, DecodeArgs* a) {
+  if (a->n_layers > kInlineLayers) return;
+  for (int i = 0; i < a->n_layers; ++i) a->inline_window[i] = h->window[a->layer_begin + i];
+}
+
 int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq_ids, const int32_t* kv_lens,
                 int batch, const void* q, void* out, int num_splits, char** error_msg) {
   if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
@@ -258,6 +263,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   a.batch = batch;
   a.num_splits = num_splits;
   a.max_kv_len = max_len;
+  fill_inline_windows(h, &a);
   HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream,
                               h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr));
   h->timed = h->timing;
@@ -334,6 +340,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.batch = n;
     a.num_splits = 1;
     a.max_kv_len = q_pos0 + n;
+    fill_inline_windows(h, &a);
     HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream, e0, e1));
   }
   h->timed = h->timing;

@@ -25,6 +25,8 @@
 
 #include "attn_params.h"
 #include "kernels.h"
+#include <hip/hip_ext.h>
+
 #include "mfma_util.h"
 
 namespace mi355 {
@@ -252,11 +254,10 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
   const int pt = 4 / hpb;
   const dim3 grid((a.n + 32 * pt - 1) / (32 * pt), a.geom.hkv * (G / hpb), a.n_layers);
-  if (ev0) (void)hipEventRecord(ev0, stream);
-  if (hpb == 4) hipLaunchKernelGGL((prefill_attn_kernel<DT, D, 4>), grid, dim3(256), 0, stream, a);
-  else if (hpb == 2) hipLaunchKernelGGL((prefill_attn_kernel<DT, D, 2>), grid, dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((prefill_attn_kernel<DT, D, 1>), grid, dim3(256), 0, stream, a);
-  if (ev1) (void)hipEventRecord(ev1, stream);
+  // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
+  if (hpb == 4) hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 4>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
+  else if (hpb == 2) hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 2>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
+  else hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 1>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
   return hipGetLastError();
 }
 
