@@ -7,5 +7,6 @@ The directory name carries a hyphen, so the package is loaded by path (see
     executor  ctypes binding of the C++ HipLlmExecutor test surface
 """
 from . import attn  # noqa: F401
+from . import executor  # noqa: F401
 
-__all__ = ["attn"]
+__all__ = ["attn", "executor"]

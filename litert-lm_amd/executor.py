@@ -1,0 +1,171 @@
+"""ctypes binding of libhip_llm_executor.so: the C++ HipLlmExecutor driven
+through its C test surface (litert-lm_amd/executor/executor_c_api.cc)."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+from . import attn as _attn
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhip_llm_executor.so")
+_lib = None
+
+
+class ExecutorError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"executor status {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class _Config(ctypes.Structure):
+    _fields_ = [
+        ("num_layers", ctypes.c_int32), ("num_q_heads", ctypes.c_int32), ("num_kv_heads", ctypes.c_int32),
+        ("vocab", ctypes.c_int32), ("max_num_tokens", ctypes.c_int32),
+        ("layer_window", ctypes.POINTER(ctypes.c_int32)),
+        ("runner_lengths", ctypes.POINTER(ctypes.c_int32)),
+        ("num_runners", ctypes.c_int32), ("fp16_activations", ctypes.c_int32),
+        ("recording_backend", ctypes.c_int32), ("execute_pending_on_single_id_chunk", ctypes.c_int32),
+        ("softcap", ctypes.c_float),
+    ]
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(f"{LIB_PATH} is missing: build it with `make -C litert-lm_amd/executor`")
+        _attn.lib()  # dependency, loaded first so that the rpath-less case still resolves
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32 = ctypes.c_void_p, ctypes.c_int32
+        i32p = ctypes.POINTER(ctypes.c_int32)
+        errp = ctypes.POINTER(ctypes.c_void_p)
+        L.hle_create.argtypes = [ctypes.POINTER(_Config), ctypes.POINTER(vp), errp]
+        L.hle_destroy.argtypes = [vp]
+        L.hle_destroy.restype = None
+        L.hle_prefill.argtypes = [vp, i32p, i32, i32, errp]
+        L.hle_decode.argtypes = [vp, i32p, errp]
+        L.hle_decode_logits.argtypes = [vp, i32, ctypes.POINTER(ctypes.c_float), errp]
+        for n in ("hle_current_step", "hle_vocab_size", "hle_max_num_tokens", "hle_num_runs"):
+            getattr(L, n).argtypes = [vp]
+        L.hle_reset.argtypes = [vp, errp]
+        L.hle_backend_name.argtypes = [vp]
+        L.hle_backend_name.restype = ctypes.c_char_p
+        L.hle_get_run.argtypes = [vp, i32, i32p, i32p, i32p, i32]
+        L.hle_backend_from_string.argtypes = [ctypes.c_char_p]
+        L.hle_plan.argtypes = [i32p, i32, i32, i32p, i32p, i32]
+        _lib = L
+    return _lib
+
+
+def _check(rc, err):
+    msg = ""
+    if err.value:
+        msg = ctypes.string_at(err.value).decode("utf-8", "replace")
+        _attn._libc.free(err.value)
+    if rc != 0:
+        raise ExecutorError(rc, msg)
+
+
+def _arr(xs):
+    xs = [int(x) for x in xs]
+    return (ctypes.c_int32 * len(xs))(*xs)
+
+
+class HipLlmExecutor:
+    """HipLlmExecutor over the synthetic decoder layers (test scaffolding)."""
+
+    def __init__(self, num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens, runner_lengths=(1024,),
+                 layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=True,
+                 softcap=0.0):
+        self._win = _arr(layer_window) if layer_window is not None else None
+        self._runners = _arr(runner_lengths)
+        cfg = _Config(num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens,
+                      ctypes.cast(self._win, ctypes.POINTER(ctypes.c_int32)) if self._win is not None else None,
+                      ctypes.cast(self._runners, ctypes.POINTER(ctypes.c_int32)), len(runner_lengths), int(fp16),
+                      int(recording_backend), int(execute_pending_on_single_id_chunk), softcap)
+        self._h = ctypes.c_void_p()
+        err = ctypes.c_void_p()
+        _check(lib().hle_create(ctypes.byref(cfg), ctypes.byref(self._h), ctypes.byref(err)), err)
+        self.vocab = vocab
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            lib().hle_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def prefill(self, ids, batch=1):
+        ids = list(ids)
+        n = len(ids) // batch if batch else 0
+        err = ctypes.c_void_p()
+        _check(lib().hle_prefill(self._h, _arr(ids), batch, n, ctypes.byref(err)), err)
+
+    def decode(self) -> int:
+        tok = ctypes.c_int32(-7)
+        err = ctypes.c_void_p()
+        _check(lib().hle_decode(self._h, ctypes.byref(tok), ctypes.byref(err)), err)
+        return tok.value
+
+    def decode_logits(self, explicit_id=None) -> np.ndarray:
+        out = np.zeros(self.vocab, dtype=np.float32)
+        err = ctypes.c_void_p()
+        _check(lib().hle_decode_logits(self._h, -1 if explicit_id is None else int(explicit_id),
+                                       out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), ctypes.byref(err)), err)
+        return out
+
+    def current_step(self) -> int:
+        return lib().hle_current_step(self._h)
+
+    def vocab_size(self) -> int:
+        return lib().hle_vocab_size(self._h)
+
+    def max_num_tokens(self) -> int:
+        return lib().hle_max_num_tokens(self._h)
+
+    def backend_name(self) -> str:
+        return lib().hle_backend_name(self._h).decode()
+
+    def reset(self):
+        err = ctypes.c_void_p()
+        _check(lib().hle_reset(self._h, ctypes.byref(err)), err)
+
+    def runs(self):
+        """[(kind, tokens, positions)] of every forward pass since the last reset."""
+        out = []
+        cap = 1 << 16
+        toks = (ctypes.c_int32 * cap)()
+        pos = (ctypes.c_int32 * cap)()
+        for i in range(lib().hle_num_runs(self._h)):
+            dec = ctypes.c_int32()
+            n = lib().hle_get_run(self._h, i, ctypes.byref(dec), toks, pos, cap)
+            out.append(("decode" if dec.value else "prefill", list(toks[:n]), list(pos[:n])))
+        return out
+
+
+def backend_from_string(s: str) -> int:
+    return lib().hle_backend_from_string(s.encode())
+
+
+def plan(runner_lengths, n):
+    cap = 4096
+    lens = (ctypes.c_int32 * cap)()
+    counts = (ctypes.c_int32 * cap)()
+    k = lib().hle_plan(_arr(runner_lengths), len(runner_lengths), n, lens, counts, cap)
+    if k < 0:
+        raise ExecutorError(-k, "plan")
+    return [(lens[i], counts[i]) for i in range(k)]

@@ -1,0 +1,88 @@
+// What the executor needs from an attention implementation: a KV cache it can
+// append rows to, and prefill / decode attention over it. Mi355AttentionBackend
+// forwards to the C ABI of libmi355_attn.so (include/mi355_attn.h);
+// RecordingAttentionBackend keeps only the call trace and returns zeros, so the
+// executor's host logic can be tested on a machine without a GPU (the same
+// role FakeLlmExecutor plays for the reference's callers,
+// runtime/executor/fake_llm_executor.h:31-91).
+#ifndef LITERT_LM_AMD_EXECUTOR_ATTENTION_BACKEND_H_
+#define LITERT_LM_AMD_EXECUTOR_ATTENTION_BACKEND_H_
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "status.h"
+
+struct mi355_attn;
+
+namespace litert::lm {
+
+struct AttentionShape {
+  int num_layers = 0;
+  int num_q_heads = 0;
+  int num_kv_heads = 0;
+  int head_dim = 256;
+  int max_tokens = 0;
+  std::vector<int> layer_window;  // per layer, 0 = global
+  float scale = 0.f;              // 0 => head_dim^-0.5
+  float softcap = 0.f;
+};
+
+class AttentionBackend {
+ public:
+  virtual ~AttentionBackend() = default;
+  // k, v: [n][kv_heads][head_dim] float32 host rows written at pos .. pos+n-1.
+  virtual Status Append(int layer, int pos, int n, const float* k, const float* v) = 0;
+  // q, out: [n][q_heads][head_dim] float32 host; rows at positions q_pos0 .. q_pos0+n-1.
+  virtual Status Prefill(int layer, int q_pos0, int n, const float* q, float* out) = 0;
+  // One row at position kv_len - 1.
+  virtual Status Decode(int layer, int kv_len, const float* q, float* out) = 0;
+  virtual Status Reset() = 0;
+  virtual std::string Name() const = 0;
+};
+
+struct AttentionCall {
+  enum Kind { kAppend, kPrefill, kDecode, kReset } kind;
+  int layer, pos, n;
+};
+
+class RecordingAttentionBackend : public AttentionBackend {
+ public:
+  explicit RecordingAttentionBackend(AttentionShape shape) : shape_(std::move(shape)) {}
+  Status Append(int layer, int pos, int n, const float*, const float*) override {
+    if (pos + n > shape_.max_tokens) return OutOfRangeError("KV cache is full.");
+    calls.push_back({AttentionCall::kAppend, layer, pos, n});
+    return OkStatus();
+  }
+  Status Prefill(int layer, int q_pos0, int n, const float*, float* out) override {
+    calls.push_back({AttentionCall::kPrefill, layer, q_pos0, n});
+    Zero(out, n);
+    return OkStatus();
+  }
+  Status Decode(int layer, int kv_len, const float*, float* out) override {
+    calls.push_back({AttentionCall::kDecode, layer, kv_len - 1, 1});
+    Zero(out, 1);
+    return OkStatus();
+  }
+  Status Reset() override {
+    calls.push_back({AttentionCall::kReset, 0, 0, 0});
+    return OkStatus();
+  }
+  std::string Name() const override { return "recording"; }
+  std::vector<AttentionCall> calls;
+
+ private:
+  void Zero(float* out, int n) const {
+    for (size_t i = 0; i < (size_t)n * shape_.num_q_heads * shape_.head_dim; ++i) out[i] = 0.f;
+  }
+  AttentionShape shape_;
+};
+
+// fp32 activations: fp32 cache and I/O. fp16 activations: fp16 cache and I/O
+// (converted on the host at this boundary).
+StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const AttentionShape& shape, bool fp16,
+                                                                         int device);
+
+}  // namespace litert::lm
+#endif  // LITERT_LM_AMD_EXECUTOR_ATTENTION_BACKEND_H_

@@ -1,0 +1,68 @@
+// Everything of the transformer that is NOT attention, as the executor sees
+// it. In the reference all of it (embedding, projections, RoPE, norms, MLP,
+// logits) sits inside the .tflite graph behind compiled_model_.Run
+// (runtime/executor/llm_litert_compiled_model_executor.cc:271,407,522); this
+// build accelerates the attention between ProjectQkv and ConsumeAttention and
+// leaves the rest to whoever implements this interface.
+//
+// SyntheticDecoderLayers is a deterministic, seed-free toy stack (hash-derived
+// embeddings and element-wise weights, RMS norm, a small logits projection)
+// used to drive the executor end to end in tests; it is test scaffolding for
+// the cache / position / step plumbing, not a model.
+#ifndef LITERT_LM_AMD_EXECUTOR_DECODER_LAYERS_H_
+#define LITERT_LM_AMD_EXECUTOR_DECODER_LAYERS_H_
+
+#include <cstdint>
+#include <vector>
+
+#include "attention_backend.h"
+#include "status.h"
+
+namespace litert::lm {
+
+class DecoderLayers {
+ public:
+  virtual ~DecoderLayers() = default;
+  virtual const AttentionShape& Shape() const = 0;
+  virtual int VocabSize() const = 0;
+  // Starts a forward pass over n tokens at the given absolute positions.
+  virtual Status Begin(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions) = 0;
+  // q [n][Hq][D], k and v [n][Hkv][D] of `layer` for the tokens of this pass.
+  virtual Status ProjectQkv(int layer, float* q, float* k, float* v) = 0;
+  // attn [n][Hq][D]: the attention output of `layer`.
+  virtual Status ConsumeAttention(int layer, const float* attn) = 0;
+  // Logits [vocab] of the last token of this pass.
+  virtual Status Logits(float* logits) = 0;
+};
+
+class SyntheticDecoderLayers : public DecoderLayers {
+ public:
+  SyntheticDecoderLayers(AttentionShape shape, int vocab) : shape_(std::move(shape)), vocab_(vocab) {}
+  const AttentionShape& Shape() const override { return shape_; }
+  int VocabSize() const override { return vocab_; }
+  Status Begin(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions) override;
+  Status ProjectQkv(int layer, float* q, float* k, float* v) override;
+  Status ConsumeAttention(int layer, const float* attn) override;
+  Status Logits(float* logits) override;
+
+  static uint32_t Mix(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7feb352dU;
+    x ^= x >> 15;
+    x *= 0x846ca68bU;
+    x ^= x >> 16;
+    return x;
+  }
+  // Uniform in [-1, 1) from a 32-bit key.
+  static float Unit(uint32_t key) { return static_cast<float>(Mix(key) >> 8) * (1.0f / 16777216.0f) * 2.0f - 1.0f; }
+
+ private:
+  int Hidden() const { return shape_.num_q_heads * shape_.head_dim; }
+  AttentionShape shape_;
+  int vocab_;
+  int n_ = 0;
+  std::vector<float> state_;  // [n][hidden]
+};
+
+}  // namespace litert::lm
+#endif  // LITERT_LM_AMD_EXECUTOR_DECODER_LAYERS_H_

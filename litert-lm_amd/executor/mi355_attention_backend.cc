@@ -1,0 +1,121 @@
+// AttentionBackend over the C ABI of libmi355_attn.so. Host float32 rows cross
+// the boundary as they are (fp32 cache) or as fp16 (fp16 cache); the library
+// stages them to the device (host_io = 1) and returns with results in place,
+// which is what the executor's synchronous Decode contract needs
+// (runtime/executor/llm_litert_compiled_model_executor.cc:528-533 hands out a
+// host-visible logits buffer right after the step).
+#include <cstdlib>
+#include <vector>
+
+#include "../../include/mi355_attn.h"
+#include "attention_backend.h"
+
+namespace litert::lm {
+namespace {
+
+Status FromCode(int rc, char* err, const char* what) {
+  if (rc == MI355_ATTN_OK) return OkStatus();
+  std::string msg = std::string(what) + ": " + (err ? err : "(no message)");
+  free(err);
+  return Status(static_cast<StatusCode>(rc), msg);
+}
+
+class Mi355AttentionBackend : public AttentionBackend {
+ public:
+  Mi355AttentionBackend(mi355_attn* h, AttentionShape shape, bool fp16) : h_(h), shape_(std::move(shape)), fp16_(fp16) {}
+  ~Mi355AttentionBackend() override { mi355_attn_destroy(h_); }
+
+  Status Append(int layer, int pos, int n, const float* k, const float* v) override {
+    char* err = nullptr;
+    const size_t count = (size_t)n * shape_.num_kv_heads * shape_.head_dim;
+    int rc;
+    if (fp16_) {
+      ToHalf(k, count, &ha_);
+      ToHalf(v, count, &hb_);
+      rc = mi355_attn_kv_append(h_, layer, 0, pos, n, ha_.data(), hb_.data(), &err);
+    } else {
+      rc = mi355_attn_kv_append(h_, layer, 0, pos, n, k, v, &err);
+    }
+    return FromCode(rc, err, "kv_append");
+  }
+
+  Status Prefill(int layer, int q_pos0, int n, const float* q, float* out) override {
+    char* err = nullptr;
+    const size_t count = (size_t)n * shape_.num_q_heads * shape_.head_dim;
+    int rc;
+    if (fp16_) {
+      ToHalf(q, count, &ha_);
+      hb_.resize(count);
+      rc = mi355_attn_prefill(h_, layer, 0, q_pos0, n, ha_.data(), hb_.data(), &err);
+      if (rc == MI355_ATTN_OK) FromHalf(hb_, count, out);
+    } else {
+      rc = mi355_attn_prefill(h_, layer, 0, q_pos0, n, q, out, &err);
+    }
+    return FromCode(rc, err, "prefill");
+  }
+
+  Status Decode(int layer, int kv_len, const float* q, float* out) override {
+    char* err = nullptr;
+    const size_t count = (size_t)shape_.num_q_heads * shape_.head_dim;
+    const int32_t len = kv_len;
+    int rc;
+    if (fp16_) {
+      ToHalf(q, count, &ha_);
+      hb_.resize(count);
+      rc = mi355_attn_decode(h_, layer, nullptr, &len, 1, ha_.data(), hb_.data(), 0, &err);
+      if (rc == MI355_ATTN_OK) FromHalf(hb_, count, out);
+    } else {
+      rc = mi355_attn_decode(h_, layer, nullptr, &len, 1, q, out, 0, &err);
+    }
+    return FromCode(rc, err, "decode");
+  }
+
+  Status Reset() override {
+    char* err = nullptr;
+    return FromCode(mi355_attn_reset(h_, -1, &err), err, "reset");
+  }
+
+  std::string Name() const override { return mi355_attn_version(); }
+
+ private:
+  static void ToHalf(const float* src, size_t n, std::vector<_Float16>* dst) {
+    dst->resize(n);
+    for (size_t i = 0; i < n; ++i) (*dst)[i] = static_cast<_Float16>(src[i]);
+  }
+  static void FromHalf(const std::vector<_Float16>& src, size_t n, float* dst) {
+    for (size_t i = 0; i < n; ++i) dst[i] = static_cast<float>(src[i]);
+  }
+  mi355_attn* h_;
+  AttentionShape shape_;
+  bool fp16_;
+  std::vector<_Float16> ha_, hb_;
+};
+
+}  // namespace
+
+StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const AttentionShape& shape, bool fp16,
+                                                                         int device) {
+  mi355_attn_config cfg{};
+  cfg.struct_size = sizeof(cfg);
+  cfg.num_layers = shape.num_layers;
+  cfg.num_q_heads = shape.num_q_heads;
+  cfg.num_kv_heads = shape.num_kv_heads;
+  cfg.head_dim = shape.head_dim;
+  cfg.max_tokens = shape.max_tokens;
+  cfg.max_seqs = 1;  // the reference executor is batch 1 (llm_litert_compiled_model_executor.cc:798-800)
+  cfg.kv_dtype = fp16 ? MI355_ATTN_F16 : MI355_ATTN_F32;
+  cfg.io_dtype = cfg.kv_dtype;
+  cfg.scale = shape.scale;
+  cfg.softcap = shape.softcap;
+  cfg.layer_window = shape.layer_window.empty() ? nullptr : shape.layer_window.data();
+  cfg.device = device;
+  cfg.host_io = 1;
+  cfg.own_stream = 1;
+  mi355_attn* h = nullptr;
+  char* err = nullptr;
+  const int rc = mi355_attn_create(&cfg, &h, &err);
+  if (rc != MI355_ATTN_OK) return FromCode(rc, err, "mi355_attn_create");
+  return std::unique_ptr<AttentionBackend>(new Mi355AttentionBackend(h, shape, fp16));
+}
+
+}  // namespace litert::lm

@@ -1,0 +1,103 @@
+"""numpy twin of SyntheticDecoderLayers (litert-lm_amd/executor/synthetic_decoder_layers.cc)
+plus a whole-sequence reference forward pass that uses the CPU oracle for
+attention. Test helper only."""
+import numpy as np
+
+from oracle import attn_oracle as orc
+
+D = 256
+M32 = np.uint64(0xFFFFFFFF)
+
+
+def mix(x):
+    x = np.asarray(x, dtype=np.uint64) & M32
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & M32
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & M32
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def unit(key):
+    key = np.asarray(key, dtype=np.uint64) & M32
+    return ((mix(key) >> np.uint64(8)).astype(np.float32) * np.float32(1.0 / 16777216.0) * np.float32(2.0)
+            - np.float32(1.0)).astype(np.float32)
+
+
+def u(x):
+    return np.asarray(x, dtype=np.uint64)
+
+
+def key(*terms):
+    acc = u(0)
+    for t in terms:
+        acc = (acc + t) & M32
+    return acc
+
+
+class Twin:
+    def __init__(self, layers, hq, hkv, vocab, windows=None, softcap=0.0):
+        self.layers, self.hq, self.hkv, self.vocab = layers, hq, hkv, vocab
+        self.windows = windows or [0] * layers
+        self.softcap = softcap
+        self.hidden = hq * D
+
+    def embed(self, tokens, positions):
+        i = u(np.arange(self.hidden))[None, :]
+        tok = u(tokens)[:, None]
+        pos = u(positions)[:, None]
+        a = unit(key(tok * u(0x9E3779B1), i * u(0x85EBCA77), u(1)))
+        b = unit(key(pos * u(0xC2B2AE3D), i * u(0x27D4EB2F), u(2)))
+        return (a + np.float32(0.5) * b).astype(np.float32)
+
+    def project(self, layer, s):
+        n = s.shape[0]
+        ul = u(layer)
+        i = u(np.arange(self.hidden))
+        wq = np.float32(1.0) + np.float32(0.5) * unit(key(ul * u(0x165667B1), i * u(0x9E3779B1), u(3)))
+        q = (s * wq[None, :]).astype(np.float32).reshape(n, self.hq, D)
+        g = self.hq // self.hkv
+        sh = s.reshape(n, self.hkv, g, D)
+        summ = np.zeros((n, self.hkv, D), np.float32)
+        for j in range(g):
+            summ = (summ + sh[:, :, j, :]).astype(np.float32)
+        mean = (summ * np.float32(1.0 / g)).astype(np.float32)
+        idx = u(np.arange(self.hkv * D)).reshape(self.hkv, D)
+        wk = np.float32(1.0) + np.float32(0.5) * unit(key(ul * u(0x27D4EB2F), idx * u(0x165667B1), u(5)))
+        k = (mean * wk[None]).astype(np.float32)
+        wv = unit(key(ul * u(0x85EBCA77), idx * u(0xC2B2AE3D), u(6)))
+        bv = np.float32(0.25) * unit(key(idx * u(0x9E3779B1), ul, u(7)))
+        v = ((mean * wv[None]).astype(np.float32) + bv[None]).astype(np.float32)
+        return q, k, v
+
+    def consume(self, layer, s, attn):
+        i = u(np.arange(self.hidden))
+        wo = unit(key(u(layer) * u(0xC2B2AE3D), i * u(0x27D4EB2F), u(8)))
+        s = (s + (attn.reshape(s.shape) * wo[None, :]).astype(np.float32)).astype(np.float32)
+        sq = (s.astype(np.float64) ** 2).sum(axis=1)
+        inv = (1.0 / np.sqrt(sq / self.hidden + 1e-6)).astype(np.float32)
+        return (s * inv[:, None]).astype(np.float32)
+
+    def logits(self, s_last):
+        i = u(np.arange(self.hidden))[None, :]
+        vv = u(np.arange(self.vocab))[:, None]
+        w = unit(key(vv * u(0x2545F491), i * u(0x61C88647), u(4))).astype(np.float64)
+        return ((w @ s_last.astype(np.float64)) / np.sqrt(self.hidden)).astype(np.float32)
+
+    def forward_all(self, tokens, round_io=None):
+        """Causal forward over the whole token list at once; returns logits of
+        every position ``[n, vocab]``. ``round_io`` (e.g. np.float16) rounds
+        q/k/v and the attention output the way a 16-bit cache does."""
+        n = len(tokens)
+        s = self.embed(tokens, np.arange(n))
+        scale = D ** -0.5
+        for layer in range(self.layers):
+            q, k, v = self.project(layer, s)
+            if round_io is not None:
+                q, k, v = (x.astype(round_io).astype(np.float32) for x in (q, k, v))
+            attn = orc.sdpa(q, k, v, scale, window=self.windows[layer], softcap=self.softcap)
+            if round_io is not None:
+                attn = attn.astype(round_io)
+            s = self.consume(layer, s, attn.astype(np.float32))
+        return np.stack([self.logits(s[t]) for t in range(n)])
