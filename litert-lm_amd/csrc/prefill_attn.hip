@@ -1,15 +1,16 @@
 // Causal / sliding-window prefill attention over the KV cache (gfx950, MFMA).
 //
-// Grid: x = tile of query positions, y = KV head x head block, z = layer.
-// A workgroup of 4 waves covers HPB query heads of one KV head times PT tiles
-// of 32 consecutive positions (HPB * PT = 4); all its waves walk the same
-// 32-key blocks, so each K/V block is brought from HBM/L2 into LDS once per
-// workgroup and read from there as MFMA operands. The key loop starts at the
-// first block the window still reaches and stops at the diagonal.
+// Grid: x = (layer, KV head, head block), y = tile of query positions, longest
+// key loops first. A workgroup of 4 waves covers HPB query heads of one KV head
+// times PT tiles of 32 consecutive positions (HPB * PT = 4); all its waves walk
+// the same 32-key blocks, so each K/V block is brought from HBM/L2 into a
+// double-buffered LDS stage once per workgroup (global_load ... lds, no
+// registers in between) and read from there as MFMA operands. The key loop starts at the first block the window still reaches
+// and stops at the diagonal.
 //
 // Per wave and key block (32x32x16 MFMA, transposed formulation so that one
 // lane owns one query):
-//   S^T[key][query] = K . Q^T        16 MFMAs (head_dim 256), Q^T in registers
+//   S^T[key][query] = K . Q^T        16 MFMAs (head_dim 256), Q^T in a per-wave LDS slice
 //   online softmax on the 16 scores a lane holds for its query
 //   O^T[d][query]  += V^T . P^T      16 MFMAs, P^T taken from S^T's registers
 // The row order in which K is fed to the first MFMA is chosen so that the
@@ -34,6 +35,7 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKeysPerBlock = 32;  // one V block of a 16-bit cache = two K tiles
+constexpr float kRescaleSlack = 8.f;  // log2 units a score may exceed the reference max before it is moved
 
 template <int T>
 struct El;
@@ -53,8 +55,13 @@ struct El<kBF16> {
 // Key (0..31, within a block) that MFMA row m of S^T stands for.
 __device__ __forceinline__ int key_of_row(int m) { return 16 * ((m >> 3) & 1) + 8 * (m >> 4) + (m & 7); }
 
+// LDS plan (dynamic): two stages of (K block, V block) then the Q^T operands
+// of the four waves: 2 * 2 * 64*D + 4 * (D/16) * 1 KiB = 128 KiB at head_dim 256.
+template <int D>
+constexpr int prefill_lds_bytes() { return 4 * 64 * D + 4 * (D / 16) * 1024; }
+
 template <int DT, int D, int HPB>
-__global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) {
+__global__ void __launch_bounds__(256, 2) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
   using vec8 = typename E::vec8;
@@ -62,46 +69,35 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) 
   constexpr int NJ = D / 16;             // K-slices of the QK^T product
   constexpr int NDP = D / 32;            // 32-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;    // one 32-key block of a 16-bit plane
-  constexpr int kChunksPerThread = kBlockBytes / 16 / 256;
+  constexpr int kStageBytes = 2 * kBlockBytes;
 
-  __shared__ __attribute__((aligned(16))) uint8_t sm_k[kBlockBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t sm_v[kBlockBytes];
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint8_t* const sm_kv = smem;                                // [2 stages][K block | V block]
+  vec8* const sm_q_all = reinterpret_cast<vec8*>(smem + 2 * kStageBytes);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, hh = lane >> 5;
+  // x = (layer, KV head, head block), y = position tile, heaviest tiles first:
+  // workgroups are dispatched x-fastest, so every layer's longest key loops
+  // start before any short one.
   const int hblocks = a.group / HPB;
-  const int kvh = blockIdx.y / hblocks, hb = blockIdx.y - kvh * hblocks;
-  const int li = blockIdx.z, layer = a.layer_begin + li;
+  const int per_layer = a.geom.hkv * hblocks;
+  const int li = blockIdx.x / per_layer, rem = blockIdx.x - li * per_layer;
+  const int kvh = rem / hblocks, hb = rem - kvh * hblocks;
+  const int tile = gridDim.y - 1 - blockIdx.y;
+  const int layer = a.layer_begin + li;
   const int window = a.layer_window[layer];
   const int head = kvh * a.group + hb * HPB + (wave % HPB);
-  const int wg_pos0 = a.q_pos0 + blockIdx.x * (32 * PT);  // first position of the workgroup
-  const int pos_end = a.q_pos0 + a.n;                     // one past the last query position
-  const int my_pos0 = wg_pos0 + (wave / HPB) * 32;        // first position of this wave's tile
-  const int row = my_pos0 - a.q_pos0 + n;                 // query row in q / out
+  const int wg_pos0 = a.q_pos0 + tile * (32 * PT);   // first position of the workgroup
+  const int pos_end = a.q_pos0 + a.n;                // one past the last query position
+  const int my_pos0 = wg_pos0 + (wave / HPB) * 32;   // first position of this wave's tile
+  const int row = my_pos0 - a.q_pos0 + n;            // query row in q / out
   const int my_pos = my_pos0 + n;
   const bool row_ok = row < a.n;
 
   const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
   const uint8_t* vplane = kplane + a.geom.plane_bytes;
-
-  // Q^T operand: lane (n, hh) holds channels 16*j + 8*hh .. +7 of its query.
-  vec8 qreg[NJ];
-  {
-    const elem_t* qrow =
-        reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + (row_ok ? row : 0)) * a.hq + head) * D;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const u4 w = *reinterpret_cast<const u4*>(qrow + 16 * j + 8 * hh);
-      qreg[j] = bit_cast<vec8>(row_ok ? w : u4{0, 0, 0, 0});
-    }
-  }
-
-  f16v acc[NDP];
-#pragma unroll
-  for (int i = 0; i < NDP; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
 
   // Key blocks the workgroup walks: from the first one the window of its first
   // row reaches to the one holding the diagonal of its last valid row.
@@ -114,120 +110,166 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) 
   if (window > 0 && my_pos0 - window + 1 > 0) my_lo = (my_pos0 - window + 1) / kKeysPerBlock;
   const int my_hi = (my_pos0 + 31) / kKeysPerBlock;
 
+  // One K/V block travels HBM/L2 -> LDS without touching registers: every wave
+  // issues 8 of the 32 wave-wide 1 KiB transfers (4 of K, 4 of V); the data of
+  // lane l lands at the stage offset of the transfer + 16 * l.
+  auto fetch_block = [&](int kb, int stage) {
+    const uint8_t* kg = kplane + (int64_t)kb * kBlockBytes + lane * 16;
+    const uint8_t* vg = vplane + (int64_t)kb * kBlockBytes + lane * 16;
+    uint8_t* dst = sm_kv + stage * kStageBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = (wave + 4 * i) * 1024;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kg + off),
+                                       (__attribute__((address_space(3))) void*)(dst + off), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vg + off),
+                                       (__attribute__((address_space(3))) void*)(dst + kBlockBytes + off), 16, 0, 0);
+    }
+  };
+  fetch_block(kb_lo, 0);
+
+  // Q^T operand in this wave's LDS slice: entry (j, lane) with lane = (n, hh)
+  // holds channels 16*j + 8*hh .. +7 of the lane's query. A lane reads back only
+  // what it wrote itself.
+  vec8* const sm_q = sm_q_all + wave * (NJ * 64) + lane;
+  {
+    const elem_t* qrow =
+        reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + (row_ok ? row : 0)) * a.hq + head) * D;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const u4 w = *reinterpret_cast<const u4*>(qrow + 16 * j + 8 * hh);
+      sm_q[j * 64] = bit_cast<vec8>(row_ok ? w : u4{0, 0, 0, 0});
+    }
+  }
+
+  f16v acc[NDP];
+#pragma unroll
+  for (int i = 0; i < NDP; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
   const float sc = a.scale, softcap = a.softcap;
 
-  u4 pre_k[kChunksPerThread], pre_v[kChunksPerThread];
-  auto prefetch = [&](int kb) {
-    const uint8_t* kg = kplane + (int64_t)kb * kBlockBytes;
-    const uint8_t* vg = vplane + (int64_t)kb * kBlockBytes;
-#pragma unroll
-    for (int i = 0; i < kChunksPerThread; ++i) {
-      pre_k[i] = *reinterpret_cast<const u4*>(kg + (tid + 256 * i) * 16);
-      pre_v[i] = *reinterpret_cast<const u4*>(vg + (tid + 256 * i) * 16);
-    }
-  };
-  auto commit = [&]() {
-#pragma unroll
-    for (int i = 0; i < kChunksPerThread; ++i) {
-      *reinterpret_cast<u4*>(sm_k + (tid + 256 * i) * 16) = pre_k[i];
-      *reinterpret_cast<u4*>(sm_v + (tid + 256 * i) * 16) = pre_v[i];
-    }
-  };
+  // LDS offsets of this lane's operands inside a stage
+  const int key_row = key_of_row(n);
+  const int k_off = (key_row >> 4) * (16 * D * 2) + (key_row & 15) * 16 + hh * 256;
+  const int v_off = kBlockBytes + (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
 
-  if (kb_lo <= kb_hi) prefetch(kb_lo);
+  __builtin_amdgcn_s_waitcnt(0);  // the first block has landed
+  __syncthreads();
+
   for (int kb = kb_lo; kb <= kb_hi; ++kb) {
-    __syncthreads();  // everyone finished reading the previous block
-    commit();
-    __syncthreads();
-    if (kb + 1 <= kb_hi) prefetch(kb + 1);
-    if (kb < my_lo || kb > my_hi) continue;
+    const int stage = (kb - kb_lo) & 1;
+    // The other stage was last read before the previous barrier: refill it now,
+    // the transfers fly during this block's arithmetic.
+    if (kb + 1 <= kb_hi) fetch_block(kb + 1, stage ^ 1);
 
-    // ---- S^T = K . Q^T
-    f16v s;
+    if (kb >= my_lo && kb <= my_hi) {
+      const uint8_t* st = sm_kv + stage * kStageBytes;
+      // ---- S^T = K . Q^T, operands read from LDS eight slices at a time
+      f16v s;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) s[e] = 0.f;
-    {
-      const int key = key_of_row(n);
-      const uint8_t* kb_base = sm_k + (key >> 4) * (16 * D * 2) + (key & 15) * 16;
+      for (int e = 0; e < 16; ++e) s[e] = 0.f;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const vec8 kop = *reinterpret_cast<const vec8*>(kb_base + (2 * j + hh) * 256);
-        s = E::mfma(kop, qreg[j], s);
+      for (int j0 = 0; j0 < NJ; j0 += 8) {
+        vec8 kop[8], qop[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          kop[j] = *reinterpret_cast<const vec8*>(st + k_off + (j0 + j) * 512);
+          qop[j] = sm_q[(j0 + j) * 64];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s = E::mfma(kop[j], qop[j], s);
       }
-    }
 
-    // ---- online softmax; this lane holds 16 keys of query n
-    const int key0 = kb * kKeysPerBlock;
-    const bool interior = (key0 + 31 <= my_pos0) && (window <= 0 || my_pos0 + 31 - key0 < window);
-    float bm = -INFINITY;
+      // V operands are requested now and arrive while the softmax runs
+      vec8 vop[2 * NDP];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float x = s[i] * sc;
-      if (softcap > 0.f) x = softcap * tanhf(x / softcap);
-      x *= kLog2e;
+      for (int dp = 0; dp < NDP; ++dp) {
+        vop[2 * dp] = *reinterpret_cast<const vec8*>(st + v_off + dp * 2048);
+        vop[2 * dp + 1] = *reinterpret_cast<const vec8*>(st + v_off + dp * 2048 + 512);
+      }
+
+      // ---- online softmax in the exp2 domain; this lane holds 16 keys of query n.
+      // The reference max m_run only moves when some score of the wave exceeds
+      // it by more than kRescaleSlack (2^8 in probability): until then p is
+      // taken against the stale max (p <= 256, harmless in fp32 / fp16 / bf16)
+      // and neither the cross-lane max nor the rescale of the 128 accumulator
+      // registers is needed. m_run is shared by the two lanes of a query.
+      if (softcap > 0.f) {
+        const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = cap2 * fast_tanh(s[i] * inv_cap);
+      } else {
+        s *= sc * kLog2e;
+      }
+      const int key0 = kb * kKeysPerBlock;
+      const bool interior = (key0 + 31 <= my_pos0) && (window <= 0 || my_pos0 + 31 - key0 < window);
       if (!interior) {
-        const int key = key0 + key_of_row(8 * (i >> 2) + 4 * hh + (i & 3));
-        const bool vis = key <= my_pos && (window <= 0 || my_pos - key < window);
-        x = vis ? x : -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + key_of_row(8 * (i >> 2) + 4 * hh + (i & 3));
+          const bool vis = key <= my_pos && (window <= 0 || my_pos - key < window);
+          s[i] = vis ? s[i] : -INFINITY;
+        }
       }
-      s[i] = x;
-      bm = fmaxf(bm, x);
-    }
-    bm = wave_xor_max(bm, 32);
-    const float m_new = fmaxf(m_run, bm);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
-    float lsum = 0.f;
+      float bm = s[0];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float p = fast_exp2(s[i] - m_use);
-      s[i] = p;
-      lsum += p;
-    }
-    l_run = l_run * alpha + lsum;
-    m_run = m_new;
-    if (__any(alpha != 1.f)) {
+      for (int i = 1; i < 16; ++i) bm = fmaxf(bm, s[i]);
+      if (__any(bm > m_run + kRescaleSlack)) {
+        bm = wave_xor_max(bm, 32);
+        const float m_new = fmaxf(m_run, bm);
+        const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
+        l_run *= alpha;
 #pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
+        for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
+        m_run = m_new;
+      }
+      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+      float lsum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i] = fast_exp2(s[i] - m_use);
+        lsum += s[i];
+      }
+      l_run += lsum;
+
+      // ---- O^T += V^T . P^T
+      if constexpr (DT == kBF16) {
+        // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
+        // them, otherwise P.V alone carries ~1e-3 of relative error.
+        vec8 p0, p1, q0, q1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p0[e] = (elem_t)s[e];
+          p1[e] = (elem_t)s[8 + e];
+          q0[e] = (elem_t)(s[e] - (float)p0[e]);
+          q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
+        }
+#pragma unroll
+        for (int dp = 0; dp < NDP; ++dp) {
+          acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
+          acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
+          acc[dp] = E::mfma(vop[2 * dp], q0, acc[dp]);
+          acc[dp] = E::mfma(vop[2 * dp + 1], q1, acc[dp]);
+        }
+      } else {
+        vec8 p0, p1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p0[e] = (elem_t)s[e];
+          p1[e] = (elem_t)s[8 + e];
+        }
+#pragma unroll
+        for (int dp = 0; dp < NDP; ++dp) {
+          acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
+          acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
+        }
+      }
     }
 
-    // ---- O^T += V^T . P^T
-    const uint8_t* vb_base = sm_v + (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
-    if constexpr (DT == kBF16) {
-      // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
-      // them, otherwise P.V alone carries ~1e-3 of relative error.
-      vec8 p0, p1, q0, q1;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p0[e] = (elem_t)s[e];
-        p1[e] = (elem_t)s[8 + e];
-        q0[e] = (elem_t)(s[e] - (float)p0[e]);
-        q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
-      }
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
-        const vec8 v0 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048);
-        const vec8 v1 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048 + 512);
-        acc[dp] = E::mfma(v0, p0, acc[dp]);
-        acc[dp] = E::mfma(v1, p1, acc[dp]);
-        acc[dp] = E::mfma(v0, q0, acc[dp]);
-        acc[dp] = E::mfma(v1, q1, acc[dp]);
-      }
-    } else {
-      vec8 p0, p1;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p0[e] = (elem_t)s[e];
-        p1[e] = (elem_t)s[8 + e];
-      }
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
-        const vec8 v0 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048);
-        const vec8 v1 = *reinterpret_cast<const vec8*>(vb_base + dp * 2048 + 512);
-        acc[dp] = E::mfma(v0, p0, acc[dp]);
-        acc[dp] = E::mfma(v1, p1, acc[dp]);
-      }
-    }
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's share of the next block has landed in LDS
+    __syncthreads();
   }
 
   // ---- normalise and store: lane (n, hh) holds channels 32*dp + 8*a + 4*hh + b
@@ -248,17 +290,30 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) 
   }
 }
 
+template <int DT, int D, int HPB>
+hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  constexpr int kLds = prefill_lds_bytes<D>();
+  static bool configured = false;  // more than 64 KiB of LDS has to be requested once per kernel
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
+  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB>), grid, dim3(256), kLds, stream, ev0, ev1, 0, a);
+  return hipGetLastError();
+}
+
 template <int DT, int D>
 hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int G = a.group;
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
   const int pt = 4 / hpb;
-  const dim3 grid((a.n + 32 * pt - 1) / (32 * pt), a.geom.hkv * (G / hpb), a.n_layers);
-  // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
-  if (hpb == 4) hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 4>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
-  else if (hpb == 2) hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 2>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
-  else hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, 1>), grid, dim3(256), 0, stream, ev0, ev1, 0, a);
-  return hipGetLastError();
+  const dim3 grid(a.n_layers * a.geom.hkv * (G / hpb), (a.n + 32 * pt - 1) / (32 * pt), 1);
+  if (hpb == 4) return launch_hpb<DT, D, 4>(a, grid, stream, ev0, ev1);
+  if (hpb == 2) return launch_hpb<DT, D, 2>(a, grid, stream, ev0, ev1);
+  return launch_hpb<DT, D, 1>(a, grid, stream, ev0, ev1);
 }
 
 }  // namespace
