@@ -4,8 +4,9 @@
 // key loops first. A workgroup of 4 waves covers HPB query heads of one KV head
 // times PT tiles of 32 consecutive positions (HPB * PT = 4); all its waves walk
 // the same 32-key blocks, so each K/V block is brought from HBM/L2 into a
-// double-buffered LDS stage once per workgroup (global_load ... lds, no
-// registers in between) and read from there as MFMA operands. The key loop starts at the first block the window still reaches
+// three-stage LDS ring once per workgroup (global_load ... lds, no registers
+// in between, two iterations ahead) and read from there as MFMA operands, the
+// K operands one block ahead of their use. The key loop starts at the first block the window still reaches
 // and stops at the diagonal.
 //
 // Per wave and key block (32x32x16 MFMA, transposed formulation so that one
@@ -55,13 +56,21 @@ struct El<kBF16> {
 // Key (0..31, within a block) that MFMA row m of S^T stands for.
 __device__ __forceinline__ int key_of_row(int m) { return 16 * ((m >> 3) & 1) + 8 * (m >> 4) + (m & 7); }
 
-// LDS plan (dynamic): two stages of (K block, V block) then the Q^T operands
-// of the four waves: 2 * 2 * 64*D + 4 * (D/16) * 1 KiB = 128 KiB at head_dim 256.
+// LDS plan (dynamic): a ring of three K blocks, a ring of three V blocks and
+// the Q^T operands of the four waves: (3 + 3) * 64*D + 4 * (D/16) KiB = 160 KiB
+// at head_dim 256, the whole LDS of a CU.
+constexpr int kStages = 3;
 template <int D>
-constexpr int prefill_lds_bytes() { return 4 * 64 * D + 4 * (D / 16) * 1024; }
+constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D + 4 * (D / 16) * 1024; }
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt[3:0], expcnt[6:4], lgkmcnt[11:8],
+// vmcnt[15:14]) that wait on vector-memory operations only.
+constexpr int kWaitVm0 = 0x0F70;  // all of this wave's transfers have landed
+constexpr int kWaitVm4 = 0x0F74;  // all but the 4 most recent ones
+constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
 
 template <int DT, int D, int HPB>
-__global__ void __launch_bounds__(256, 2) prefill_attn_kernel(const PrefillArgs a) {
+__global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
   using vec8 = typename E::vec8;
@@ -69,11 +78,11 @@ __global__ void __launch_bounds__(256, 2) prefill_attn_kernel(const PrefillArgs 
   constexpr int NJ = D / 16;             // K-slices of the QK^T product
   constexpr int NDP = D / 32;            // 32-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;    // one 32-key block of a 16-bit plane
-  constexpr int kStageBytes = 2 * kBlockBytes;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* const sm_kv = smem;                                // [2 stages][K block | V block]
-  vec8* const sm_q_all = reinterpret_cast<vec8*>(smem + 2 * kStageBytes);
+  uint8_t* const sm_k = smem;                              // [kStages][K block]
+  uint8_t* const sm_v = smem + kStages * kBlockBytes;      // [kStages][V block]
+  vec8* const sm_q_all = reinterpret_cast<vec8*>(smem + 2 * kStages * kBlockBytes);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -100,33 +109,36 @@ __global__ void __launch_bounds__(256, 2) prefill_attn_kernel(const PrefillArgs 
   const uint8_t* vplane = kplane + a.geom.plane_bytes;
 
   // Key blocks the workgroup walks: from the first one the window of its first
-  // row reaches to the one holding the diagonal of its last valid row.
+  // row reaches to the one holding the diagonal of its last valid row. Every
+  // wave walks all of them (blocks outside its own tile's range are masked).
   const int last_pos = min(wg_pos0 + 32 * PT, pos_end) - 1;
   int kb_lo = 0;
   if (window > 0 && wg_pos0 - window + 1 > 0) kb_lo = (wg_pos0 - window + 1) / kKeysPerBlock;
-  const int kb_hi = last_pos / kKeysPerBlock;  // inclusive
-  // Blocks this wave needs (others are skipped without touching its state).
-  int my_lo = 0;
-  if (window > 0 && my_pos0 - window + 1 > 0) my_lo = (my_pos0 - window + 1) / kKeysPerBlock;
-  const int my_hi = (my_pos0 + 31) / kKeysPerBlock;
+  const int nblk = last_pos / kKeysPerBlock - kb_lo + 1;
 
-  // One K/V block travels HBM/L2 -> LDS without touching registers: every wave
-  // issues 8 of the 32 wave-wide 1 KiB transfers (4 of K, 4 of V); the data of
+  // A K or V block travels HBM/L2 -> LDS without touching registers: every
+  // wave issues 4 of the 16 wave-wide 1 KiB transfers of a block; the data of
   // lane l lands at the stage offset of the transfer + 16 * l.
-  auto fetch_block = [&](int kb, int stage) {
-    const uint8_t* kg = kplane + (int64_t)kb * kBlockBytes + lane * 16;
-    const uint8_t* vg = vplane + (int64_t)kb * kBlockBytes + lane * 16;
-    uint8_t* dst = sm_kv + stage * kStageBytes;
+  auto fetch = [&](const uint8_t* plane, uint8_t* ring, int i) {
+    const uint8_t* g = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16;
+    uint8_t* dst = ring + (i % kStages) * kBlockBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int off = (wave + 4 * i) * 1024;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kg + off),
+    for (int t = 0; t < 4; ++t) {
+      const int off = (wave + 4 * t) * 1024;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + off),
                                        (__attribute__((address_space(3))) void*)(dst + off), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vg + off),
-                                       (__attribute__((address_space(3))) void*)(dst + kBlockBytes + off), 16, 0, 0);
     }
   };
-  fetch_block(kb_lo, 0);
+  // Ring protocol. Iteration i requests K block i+3 and V block i+2: the stage
+  // of K(i+3) held K(i), whose operands went to registers during iteration
+  // i-1; the stage of V(i+2) held V(i-1). At the bottom of iteration i every
+  // wave waits for its share of K(i+2) and V(i+1) (requested one iteration
+  // earlier), so after the barrier iteration i+1 finds V(i+1) and K(i+2)
+  // resident: every transfer has two iterations to land.
+  fetch(kplane, sm_k, 0);
+  fetch(vplane, sm_v, 0);
+  if (nblk > 1) { fetch(kplane, sm_k, 1); fetch(vplane, sm_v, 1); }
+  if (nblk > 2) fetch(kplane, sm_k, 2);
 
   // Q^T operand in this wave's LDS slice: entry (j, lane) with lane = (n, hh)
   // holds channels 16*j + 8*hh .. +7 of the lane's query. A lane reads back only
@@ -150,125 +162,151 @@ __global__ void __launch_bounds__(256, 2) prefill_attn_kernel(const PrefillArgs 
   float m_run = -INFINITY, l_run = 0.f;
   const float sc = a.scale, softcap = a.softcap;
 
-  // LDS offsets of this lane's operands inside a stage
+  // LDS offsets of this lane's operands inside a block
   const int key_row = key_of_row(n);
   const int k_off = (key_row >> 4) * (16 * D * 2) + (key_row & 15) * 16 + hh * 256;
-  const int v_off = kBlockBytes + (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
+  const int v_off = (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
 
-  __builtin_amdgcn_s_waitcnt(0);  // the first block has landed
-  __syncthreads();
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();  // the first blocks are resident
 
-  for (int kb = kb_lo; kb <= kb_hi; ++kb) {
-    const int stage = (kb - kb_lo) & 1;
-    // The other stage was last read before the previous barrier: refill it now,
-    // the transfers fly during this block's arithmetic.
-    if (kb + 1 <= kb_hi) fetch_block(kb + 1, stage ^ 1);
+  // Operand registers: all K slices of the coming block and the first half of
+  // the Q slices are read one phase ahead of their MFMAs.
+  vec8 kop[NJ], qa[NJ / 2], qb[NJ / 2], vop[2 * NDP];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) kop[j] = *reinterpret_cast<const vec8*>(sm_k + k_off + j * 512);
+#pragma unroll
+  for (int j = 0; j < NJ / 2; ++j) qa[j] = sm_q[j * 64];
 
-    if (kb >= my_lo && kb <= my_hi) {
-      const uint8_t* st = sm_kv + stage * kStageBytes;
-      // ---- S^T = K . Q^T, operands read from LDS eight slices at a time
-      f16v s;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) s[e] = 0.f;
-#pragma unroll
-      for (int j0 = 0; j0 < NJ; j0 += 8) {
-        vec8 kop[8], qop[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          kop[j] = *reinterpret_cast<const vec8*>(st + k_off + (j0 + j) * 512);
-          qop[j] = sm_q[(j0 + j) * 64];
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s = E::mfma(kop[j], qop[j], s);
-      }
+  for (int i = 0; i < nblk; ++i) {
+    const bool fetch_k = i + 3 < nblk, fetch_v = i + 2 < nblk;
+    if (fetch_k) fetch(kplane, sm_k, i + 3);
+    if (fetch_v) fetch(vplane, sm_v, i + 2);
 
-      // V operands are requested now and arrive while the softmax runs
-      vec8 vop[2 * NDP];
+    // ---- S^T = K . Q^T; the second half of the Q slices arrives under the
+    // first eight MFMAs
+#pragma unroll
+    for (int j = 0; j < NJ / 2; ++j) qb[j] = sm_q[(NJ / 2 + j) * 64];
+    f16v s;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ / 2; ++j) s = E::mfma(kop[j], qa[j], s);
+#pragma unroll
+    for (int j = 0; j < NJ / 2; ++j) s = E::mfma(kop[NJ / 2 + j], qb[j], s);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // V operands of this block are requested now and arrive while the softmax runs
+    {
+      const uint8_t* vb = sm_v + (i % kStages) * kBlockBytes + v_off;
 #pragma unroll
       for (int dp = 0; dp < NDP; ++dp) {
-        vop[2 * dp] = *reinterpret_cast<const vec8*>(st + v_off + dp * 2048);
-        vop[2 * dp + 1] = *reinterpret_cast<const vec8*>(st + v_off + dp * 2048 + 512);
+        vop[2 * dp] = *reinterpret_cast<const vec8*>(vb + dp * 2048);
+        vop[2 * dp + 1] = *reinterpret_cast<const vec8*>(vb + dp * 2048 + 512);
       }
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
-      // ---- online softmax in the exp2 domain; this lane holds 16 keys of query n.
-      // The reference max m_run only moves when some score of the wave exceeds
-      // it by more than kRescaleSlack (2^8 in probability): until then p is
-      // taken against the stale max (p <= 256, harmless in fp32 / fp16 / bf16)
-      // and neither the cross-lane max nor the rescale of the 128 accumulator
-      // registers is needed. m_run is shared by the two lanes of a query.
-      if (softcap > 0.f) {
-        const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
+    // ---- online softmax in the exp2 domain; this lane holds 16 keys of query n.
+    // The reference max m_run only moves when some score of the wave exceeds
+    // it by more than kRescaleSlack (2^8 in probability): until then p is
+    // taken against the stale max (p <= 256, harmless in fp32 / fp16 / bf16)
+    // and neither the cross-lane max nor the rescale of the 128 accumulator
+    // registers is needed. m_run is shared by the two lanes of a query.
+    if (softcap > 0.f) {
+      const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = cap2 * fast_tanh(s[i] * inv_cap);
-      } else {
-        s *= sc * kLog2e;
+      for (int e = 0; e < 16; ++e) s[e] = cap2 * fast_tanh(s[e] * inv_cap);
+    } else {
+      s *= sc * kLog2e;
+    }
+    const int key0 = (kb_lo + i) * kKeysPerBlock;
+    const bool interior = (key0 + 31 <= my_pos0) && (window <= 0 || my_pos0 + 31 - key0 < window);
+    if (!interior) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int key = key0 + key_of_row(8 * (e >> 2) + 4 * hh + (e & 3));
+        const bool vis = key <= my_pos && (window <= 0 || my_pos - key < window);
+        s[e] = vis ? s[e] : -INFINITY;
       }
-      const int key0 = kb * kKeysPerBlock;
-      const bool interior = (key0 + 31 <= my_pos0) && (window <= 0 || my_pos0 + 31 - key0 < window);
-      if (!interior) {
+    }
+    float bm = s[0];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + key_of_row(8 * (i >> 2) + 4 * hh + (i & 3));
-          const bool vis = key <= my_pos && (window <= 0 || my_pos - key < window);
-          s[i] = vis ? s[i] : -INFINITY;
-        }
-      }
-      float bm = s[0];
+    for (int e = 1; e < 16; ++e) bm = fmaxf(bm, s[e]);
+    if (__any(bm > m_run + kRescaleSlack)) {
+      bm = wave_xor_max(bm, 32);
+      const float m_new = fmaxf(m_run, bm);
+      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
+      l_run *= alpha;
+      // The accumulators live in AGPRs (the MFMAs read and write them there);
+      // the two pins keep their detour through VGPRs inside this rare block.
 #pragma unroll
-      for (int i = 1; i < 16; ++i) bm = fmaxf(bm, s[i]);
-      if (__any(bm > m_run + kRescaleSlack)) {
-        bm = wave_xor_max(bm, 32);
-        const float m_new = fmaxf(m_run, bm);
-        const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
-        l_run *= alpha;
+      for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
 #pragma unroll
-        for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
-        m_run = m_new;
-      }
-      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-      float lsum = 0.f;
+      for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] = fast_exp2(s[i] - m_use);
-        lsum += s[i];
-      }
-      l_run += lsum;
+      for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
+      m_run = m_new;
+    }
+    const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+    float lsum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = fast_exp2(s[e] - m_use);
+      lsum += s[e];
+    }
+    l_run += lsum;
 
-      // ---- O^T += V^T . P^T
-      if constexpr (DT == kBF16) {
-        // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
-        // them, otherwise P.V alone carries ~1e-3 of relative error.
-        vec8 p0, p1, q0, q1;
+    // K operands of the next block (resident since the previous barrier) and
+    // the first half of the Q slices are requested now and arrive during P.V
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 1 < nblk) {
+      const uint8_t* nx = sm_k + ((i + 1) % kStages) * kBlockBytes + k_off;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          p0[e] = (elem_t)s[e];
-          p1[e] = (elem_t)s[8 + e];
-          q0[e] = (elem_t)(s[e] - (float)p0[e]);
-          q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
-        }
+      for (int j = 0; j < NJ; ++j) kop[j] = *reinterpret_cast<const vec8*>(nx + j * 512);
 #pragma unroll
-        for (int dp = 0; dp < NDP; ++dp) {
-          acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
-          acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
-          acc[dp] = E::mfma(vop[2 * dp], q0, acc[dp]);
-          acc[dp] = E::mfma(vop[2 * dp + 1], q1, acc[dp]);
-        }
-      } else {
-        vec8 p0, p1;
+      for (int j = 0; j < NJ / 2; ++j) qa[j] = sm_q[j * 64];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- O^T += V^T . P^T
+    if constexpr (DT == kBF16) {
+      // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
+      // them, otherwise P.V alone carries ~1e-3 of relative error.
+      vec8 p0, p1, q0, q1;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          p0[e] = (elem_t)s[e];
-          p1[e] = (elem_t)s[8 + e];
-        }
+      for (int e = 0; e < 8; ++e) {
+        p0[e] = (elem_t)s[e];
+        p1[e] = (elem_t)s[8 + e];
+        q0[e] = (elem_t)(s[e] - (float)p0[e]);
+        q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
+      }
 #pragma unroll
-        for (int dp = 0; dp < NDP; ++dp) {
-          acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
-          acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
-        }
+      for (int dp = 0; dp < NDP; ++dp) {
+        acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
+        acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
+        acc[dp] = E::mfma(vop[2 * dp], q0, acc[dp]);
+        acc[dp] = E::mfma(vop[2 * dp + 1], q1, acc[dp]);
+      }
+    } else {
+      vec8 p0, p1;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p0[e] = (elem_t)s[e];
+        p1[e] = (elem_t)s[8 + e];
+      }
+#pragma unroll
+      for (int dp = 0; dp < NDP; ++dp) {
+        acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
+        acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
       }
     }
 
-    __builtin_amdgcn_s_waitcnt(0);  // this wave's share of the next block has landed in LDS
+    // this wave's shares of K(i+2) and V(i+1) have landed; what was requested
+    // in this iteration may still be in flight
+    if (fetch_k) __builtin_amdgcn_s_waitcnt(kWaitVm8);
+    else if (fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm4);
+    else __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
   }
 
