@@ -180,7 +180,8 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
 
 /*
  * Tuning and cross-check switches (return kInvalidArgument for unknown names):
- *   "decode_waves"     1, 2 or 4 waves per decode workgroup
+ *   "decode_waves"     1, 2 or 4 waves per decode workgroup, 0 (default) = chosen
+ *                      from the number of workgroups of the launch
  *   "rowwise_prefill"  0/1 run prefill row by row through the decode kernel
  *                      (the only path for fp32 and int8 caches)
  */

@@ -428,8 +428,16 @@ hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev
 
 template <int KV, int IO, int D>
 hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t s, hipEvent_t e0, hipEvent_t e1) {
-  if (t.waves == 1) return launch_variant<KV, IO, D, 1>(a, s, e0, e1);
-  if (t.waves == 2) return launch_variant<KV, IO, D, 2>(a, s, e0, e1);
+  int waves = t.waves;
+  if (waves == 0) {
+    // Measured on MI355X (head_dim 256, 4096-token context): with several
+    // workgroups per CU one wave each is as fast or faster (fewer LDS merges),
+    // with less than one per CU more waves per workgroup hide the latency.
+    const int wgs = a.n_layers * a.batch * a.geom.hkv * a.num_splits;
+    waves = wgs >= 768 ? 1 : wgs >= 256 ? 2 : 4;
+  }
+  if (waves == 1) return launch_variant<KV, IO, D, 1>(a, s, e0, e1);
+  if (waves == 2) return launch_variant<KV, IO, D, 2>(a, s, e0, e1);
   return launch_variant<KV, IO, D, 4>(a, s, e0, e1);
 }
 

@@ -10,7 +10,7 @@
 namespace mi355 {
 
 struct DecodeTuning {
-  int waves = 2;  // waves per workgroup: 1, 2 or 4
+  int waves = 0;  // waves per workgroup: 1, 2 or 4; 0 picks by workgroup count
 };
 
 bool decode_supported(int kv_dtype, int io_dtype, int head_dim);

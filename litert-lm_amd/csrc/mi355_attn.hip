@@ -622,7 +622,7 @@ float mi355_attn_last_kernel_ms(mi355_attn* h) {
 int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   if (!h || !name) return MI355_ATTN_INVALID_ARGUMENT;
   if (!strcmp(name, "decode_waves")) {
-    if (value != 1 && value != 2 && value != 4) return MI355_ATTN_INVALID_ARGUMENT;
+    if (value != 0 && value != 1 && value != 2 && value != 4) return MI355_ATTN_INVALID_ARGUMENT;
     h->tuning.waves = value;
   } else if (!strcmp(name, "rowwise_prefill")) {
     h->rowwise_prefill = value != 0;
