@@ -145,13 +145,14 @@ def prefill_flops(n, hq, window):
     return 4 * hq * D * pairs
 
 
-def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024):
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False):
     hq, hkv = 4, 1
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
     stream = torch.cuda.current_stream().cuda_stream
-    at = A.Attn(layers, hq, hkv, D, n, 1, A.BF16, A.BF16, layer_window=windows, stream=stream)
-    fill_cache(at, torch, layers, [n], hkv, torch.bfloat16, seed=0xC0FFEE + 1)
-    q = torch.randn((layers, n, hq, D), device="cuda:0").bfloat16()
+    dt, tdt = (A.F16, torch.float16) if half else (A.BF16, torch.bfloat16)
+    at = A.Attn(layers, hq, hkv, D, n, 1, dt, dt, layer_window=windows, stream=stream)
+    fill_cache(at, torch, layers, [n], hkv, tdt, seed=0xC0FFEE + 1)
+    q = torch.randn((layers, n, hq, D), device="cuda:0").to(tdt)
     out = torch.empty_like(q)
 
     def step(i):
@@ -165,12 +166,52 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024):
         at.prefill(5, 0, 0, n, q[5], out[5])  # one global layer
     lat1 = time_steps(torch, step1, 50, 5)
     at.close()
-    return {"workload": "C2: 26 layers x 1024 tokens, Hq4/Hkv1, bf16, 22 local(W=512)+4 global, one launch",
+    return {"workload": f"C2: 26 layers x 1024 tokens, Hq4/Hkv1, {'fp16' if half else 'bf16'}, "
+                        "22 local(W=512)+4 global, one launch",
             "ms_per_step": sec * 1e3, "kernel_ms": kms, "flops": flops, "TFLOPs": flops / sec / 1e12,
             "kernel_TFLOPs": flops / (kms * 1e-3) / 1e12,
             "frac_of_mfma_peak": flops / (kms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
             "tokens_per_s": n / sec, "single_global_layer_ms": lat1 * 1e3,
             "dense_counted_TFLOPs": layers * 4 * hq * D * n * n / sec / 1e12}
+
+
+def bench_decode_c1(A, torch, steps, warmup):
+    """Config 1: fp32 cache, one sequence of 1024 tokens, Hq4/Hkv1, one layer
+    (2 MiB: a latency figure, the cache stays in L2)."""
+    hq, hkv, ctx = 4, 1, 1024
+    stream = torch.cuda.current_stream().cuda_stream
+    at = A.Attn(1, hq, hkv, D, ctx, 1, A.F32, A.F32, stream=stream)
+    fill_cache(at, torch, 1, [ctx], hkv, torch.float32, seed=0xC0FFEE)
+    q = torch.randn((1, hq, D), device="cuda:0")
+    out = torch.empty_like(q)
+    lens = A._i32_array([ctx])
+
+    def step(i):
+        at.decode(0, lens, q, out, num_splits=0, batch=1)
+
+    sec = time_steps(torch, step, steps, warmup)
+    kms = kernel_ms(torch, at, step, min(steps, 30), 0)
+    at.close()
+    nbytes = ctx * hkv * D * 2 * 4 + 2 * hq * D * 4
+    return {"workload": "C1: 1 seq x 1024, Hq4/Hkv1, fp32, one layer, cache-resident (latency)",
+            "ms_per_step": sec * 1e3, "kernel_ms": kms, "bytes": nbytes, "GBps": nbytes / sec / 1e9,
+            "kernel_GBps": nbytes / (kms * 1e-3) / 1e9, "tokens_per_s": 1.0 / sec}
+
+
+def gemm_probe(torch, n=8192, reps=20):
+    """Dense bf16 GEMM through the vendor library: what the matrix cores of this
+    very card sustain next to the published peak the roofline is priced on."""
+    a = torch.randn((n, n), device="cuda:0").bfloat16()
+    b = torch.randn((n, n), device="cuda:0").bfloat16()
+    for _ in range(3):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / reps
+    return 2 * n ** 3 / sec / 1e12
 
 
 def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=12.0):
@@ -278,6 +319,16 @@ def main():
                          "frac": round(pre["frac_of_mfma_peak"], 4), "traffic": None,
                          "algorithmic_flops_per_launch": pre["flops"], "avg_kernel_us": round(pre["kernel_ms"] * 1e3, 2)},
         }
+        pre16 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), half=True)
+        log(f"[bench] prefill C2 in fp16: {pre16['ms_per_step']:.3f} ms/step, {pre16['kernel_TFLOPs']:.1f} TFLOP/s kernel")
+        result["prefill_fp16"] = {"workload": pre16["workload"], "value": round(pre16["TFLOPs"], 2), "unit": "TFLOP/s",
+                                  "kernel_TFLOPs": round(pre16["kernel_TFLOPs"], 2),
+                                  "frac_of_mfma_peak": round(pre16["frac_of_mfma_peak"], 4),
+                                  "avg_kernel_us": round(pre16["kernel_ms"] * 1e3, 2)}
+        probe = gemm_probe(torch)
+        log(f"[bench] vendor bf16 GEMM 8192^3: {probe:.0f} TFLOP/s")
+        result["mfma_peak_probe"] = {"what": "torch.matmul bf16 8192x8192x8192 (hipBLASLt)", "TFLOPs": round(probe, 1),
+                                     "published_dense_peak_TFLOPs": MFMA_BF16_PEAK_TFLOPS}
         rng = np.random.default_rng(0xC0FFEE + 3)
         lens4 = [int(x) for x in rng.integers(256, 4097, size=64)]
         extras = []
@@ -286,6 +337,9 @@ def main():
             r = bench_decode_batch(A, torch, name, kv, lens, max(20, args.steps // 4), max(5, args.warmup // 4), rot, 16)
             log(f"[bench] {name}: {r['ms_per_step']*1e3:.1f} us/step, kernel {r['kernel_GBps']:.0f} GB/s")
             extras.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
+        c1 = bench_decode_c1(A, torch, args.steps, args.warmup)
+        log(f"[bench] {c1['workload']}: {c1['ms_per_step']*1e3:.1f} us/step")
+        extras.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in c1.items()})
         result["other_decode_configs"] = extras
 
     if not args.no_cpu:

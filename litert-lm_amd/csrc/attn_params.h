@@ -40,7 +40,7 @@ MI355_HD int dtype_size(int dt) { return dt == kF32 ? 4 : (dt == kI8 ? 1 : 2); }
 
 constexpr int kTokenAlign = 64;  // planes hold a multiple of 64 rows
 constexpr int kMaxGroup = 16;    // query heads per KV head handled by one MFMA column block
-constexpr int kInlineItems = 8;  // batches up to this size need no upload of their lengths
+constexpr int kInlineItems = 64; // batches up to this size need no upload of their lengths
 constexpr int kMaxDecodeSplits = 256;
 constexpr int kInlineLayers = 64;  // calls over up to this many layers carry their windows in the argument block
 

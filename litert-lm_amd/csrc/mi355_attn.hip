@@ -234,9 +234,9 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   HIP_OR_RETURN(hipSetDevice(h->device));
   const int items = n_layers * batch;
   if (num_splits == 0) {
-    // enough workgroups to cover the chip a few times, partitions of >= 128 tokens
+    // enough workgroups to cover the chip a few times, partitions of >= 64 tokens
     const int want = (2048 + items * h->cfg.num_kv_heads - 1) / (items * h->cfg.num_kv_heads);
-    num_splits = std::max(1, std::min({want, (max_len + 127) / 128, 64}));
+    num_splits = std::max(1, std::min({want, (max_len + 63) / 64, 64}));
   }
   DecodeArgs a{};
   if (num_splits > 1)
