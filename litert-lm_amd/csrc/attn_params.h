@@ -124,12 +124,15 @@ struct PrefillArgs {
   const uint8_t* cache;
   const float* scales;
   const int32_t* layer_window;
+  int32_t* sched;  // kPrefillSchedInts work-queue counters, all zero between launches
   CacheGeom geom;
   int32_t hq, group;
   int32_t layer_begin, n_layers;
   int32_t seq, q_pos0, n;
   float scale, softcap;
 };
+constexpr int kPrefillQueues = 8;                     // one per XCD
+constexpr int kPrefillSchedInts = kPrefillQueues + 1;  // + count of workgroups that are done
 
 struct KvCopyArgs {
   uint8_t* cache;

@@ -69,6 +69,7 @@ struct mi355_attn {
   uint64_t cache_bytes = 0;
   float* scales = nullptr;
   int32_t* d_window = nullptr;
+  int32_t* d_sched = nullptr;  // prefill work-queue counters
   std::vector<int32_t> window;
   std::vector<int32_t> filled;  // [layer][seq] rows written since the last reset
   // split-KV workspace
@@ -299,6 +300,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.cache = h->cache;
     a.scales = h->scales;
     a.layer_window = h->d_window;
+    a.sched = h->d_sched;
     a.geom = h->geom;
     a.hq = h->cfg.num_q_heads;
     a.group = h->cfg.num_q_heads / h->cfg.num_kv_heads;
@@ -445,6 +447,10 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
   if ((e = hipMemcpyAsync(h->d_window, h->window.data(), sizeof(int32_t) * c->num_layers, hipMemcpyHostToDevice,
                           h->stream)) != hipSuccess)
     return bail(MI355_ATTN_INTERNAL, "window upload", e);
+  if ((e = hipMalloc(&h->d_sched, sizeof(int32_t) * kPrefillSchedInts)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "prefill queue counters", e);
+  if ((e = hipMemsetAsync(h->d_sched, 0, sizeof(int32_t) * kPrefillSchedInts, h->stream)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "prefill queue clear", e);
   h->ring_slot_ints = 2 * c->max_seqs;
   if ((e = hipHostMalloc(&h->h_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)
     return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "pinned ring", e);
@@ -467,6 +473,7 @@ void mi355_attn_destroy(mi355_attn* h) {
   if (h->cache) (void)hipFree(h->cache);
   if (h->scales) (void)hipFree(h->scales);
   if (h->d_window) (void)hipFree(h->d_window);
+  if (h->d_sched) (void)hipFree(h->d_sched);
   if (h->ws_acc) (void)hipFree(h->ws_acc);
   if (h->ws_ml) (void)hipFree(h->ws_ml);
   if (h->d_ring) (void)hipFree(h->d_ring);

@@ -1,21 +1,26 @@
 // Causal / sliding-window prefill attention over the KV cache (gfx950, MFMA).
 //
-// Grid: x = (layer, KV head, head block), y = tile of query positions, longest
-// key loops first. A workgroup of 4 waves covers HPB query heads of one KV head
-// times PT tiles of 32 consecutive positions (HPB * PT = 4); all its waves walk
-// the same 32-key blocks, so each K/V block is brought from HBM/L2 into a
-// three-stage LDS ring once per workgroup (global_load ... lds, no registers
-// in between, two iterations ahead) and read from there as MFMA operands, the
-// K operands one block ahead of their use. The key loop starts at the first block the window still reaches
-// and stops at the diagonal.
+// A workgroup of 4 waves (one per SIMD) covers HPB query heads of one KV head
+// times PT stretches of 64 consecutive positions (HPB * PT = 4); each wave owns
+// one head and one stretch = two tiles of 32 queries. All waves walk the same
+// 32-key blocks, so each K/V block is brought from HBM/L2 into an LDS ring once
+// per workgroup (global_load ... lds, no registers in between, one iteration
+// ahead), and every K or V operand a wave reads from LDS feeds two MFMAs, one
+// per tile. The key loop starts at the first block the window still reaches and
+// stops at the diagonal.
 //
-// Per wave and key block (32x32x16 MFMA, transposed formulation so that one
-// lane owns one query):
-//   S^T[key][query] = K . Q^T        16 MFMAs (head_dim 256), Q^T in a per-wave LDS slice
+// Per wave, key block and tile (32x32x16 MFMA, transposed formulation so that
+// one lane owns one query):
+//   S^T[key][query] = K . Q^T        16 MFMAs (head_dim 256); Q^T of the first tile
+//                                    in registers, of the second in a per-wave LDS slice
 //   online softmax on the 16 scores a lane holds for its query
 //   O^T[d][query]  += V^T . P^T      16 MFMAs, P^T taken from S^T's registers
 // The row order in which K is fed to the first MFMA is chosen so that the
-// probabilities already sit in the token order of the V plane.
+// probabilities already sit in the token order of the V plane. The two tiles'
+// 256 accumulator registers fill the AGPR half of the register file.
+//
+// Work distribution: persistent workgroups, one per CU, draw (unit, stretch)
+// items from per-XCD queues of atomic tickets, longest key loops first.
 //
 // Replaces the prefill-time attention the reference reaches through
 // compiled_model_.Run(prefill_signature, ...)
@@ -24,6 +29,9 @@
 // (runtime/executor/litert_compiled_model_executor_utils.cc:332-397).
 #include <hip/hip_runtime.h>
 #include <math.h>
+
+#include <type_traits>
+#include <utility>
 
 #include "attn_params.h"
 #include "kernels.h"
@@ -56,12 +64,11 @@ struct El<kBF16> {
 // Key (0..31, within a block) that MFMA row m of S^T stands for.
 __device__ __forceinline__ int key_of_row(int m) { return 16 * ((m >> 3) & 1) + 8 * (m >> 4) + (m & 7); }
 
-// LDS plan (dynamic): a ring of three K blocks, a ring of three V blocks and
-// the Q^T operands of the four waves: (3 + 3) * 64*D + 4 * (D/16) KiB = 160 KiB
-// at head_dim 256, the whole LDS of a CU.
+// LDS plan (dynamic): a ring of three K blocks and a ring of three V blocks,
+// 2 * 3 * 64*D bytes = 96 KiB at head_dim 256.
 constexpr int kStages = 3;
 template <int D>
-constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D + 4 * (D / 16) * 1024; }
+constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D; }
 
 // s_waitcnt immediates (gfx9 encoding: vmcnt[3:0], expcnt[6:4], lgkmcnt[11:8],
 // vmcnt[15:14]) that wait on vector-memory operations only.
@@ -69,278 +76,416 @@ constexpr int kWaitVm0 = 0x0F70;  // all of this wave's transfers have landed
 constexpr int kWaitVm4 = 0x0F74;  // all but the 4 most recent ones
 constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
 
-template <int DT, int D, int HPB>
-__global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillArgs a) {
+constexpr int kWaves = 4;       // per workgroup
+constexpr int kStretch = 32;    // query positions per wave: one tile
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <int DT, int D, int HPB, bool CAP>
+__global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
   using vec8 = typename E::vec8;
-  constexpr int PT = 4 / HPB;            // position tiles per workgroup
+  constexpr int PT = 4 / HPB;            // stretches per workgroup
   constexpr int NJ = D / 16;             // K-slices of the QK^T product
   constexpr int NDP = D / 32;            // 32-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;    // one 32-key block of a 16-bit plane
+  constexpr int kXfers = 16 / kWaves;    // 1 KiB transfers per wave, block and plane
+  constexpr int NP = DT == kBF16 ? 4 : 2;  // P operands per tile: p0, p1 (+ low parts for bf16)
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint8_t* const sm_k = smem;                              // [kStages][K block]
   uint8_t* const sm_v = smem + kStages * kBlockBytes;      // [kStages][V block]
-  vec8* const sm_q_all = reinterpret_cast<vec8*>(smem + 2 * kStages * kBlockBytes);
+  // The ticket of the next work item is passed through the last V stage, which
+  // no transfer writes before the second barrier of an item.
+  volatile int* const sm_ticket = reinterpret_cast<volatile int*>(sm_v + (kStages - 1) * kBlockBytes);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, hh = lane >> 5;
-  // x = (layer, KV head, head block), y = position tile, heaviest tiles first:
-  // workgroups are dispatched x-fastest, so every layer's longest key loops
-  // start before any short one.
+  // Persistent workgroups, one per CU, draw work items = (unit, stretch) from
+  // queues of atomic tickets. A unit = (layer, KV head, head block) shares one
+  // K/V plane. Workgroup k runs on XCD k % 8 (round-robin dispatch) and each XCD
+  // has its own L2, so there is one queue per XCD holding every eighth unit, all
+  // stretches of those units, longest key loops first: the K/V blocks a CU asks
+  // for are then mostly in its XCD's L2 already. A workgroup whose own queue has
+  // run dry takes from the others', which evens out the tail.
   const int hblocks = a.group / HPB;
   const int per_layer = a.geom.hkv * hblocks;
-  const int li = blockIdx.x / per_layer, rem = blockIdx.x - li * per_layer;
+  const int units = a.n_layers * per_layer;
+  const int tiles = (a.n + kStretch * PT - 1) / (kStretch * PT);
+  const int home = blockIdx.x & (kPrefillQueues - 1);
+  int tried = 0;  // queues this workgroup has found empty (kept by thread 0)
+  const float softcap = a.softcap;  // CAP: > 0, scores go through softcap * tanh(score / softcap)
+  const float c = CAP ? 1.f : a.scale * kLog2e;
+  const int pos_end = a.q_pos0 + a.n;                // one past the last query position
+  // LDS offsets of this lane's operands inside a block
+  const int key_row = key_of_row(n);
+  const int k_off = (key_row >> 4) * (16 * D * 2) + (key_row & 15) * 16 + hh * 256;
+  const int v_off = (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
+  constexpr int kAhead = 4;  // K operand reads in flight ahead of their MFMAs
+
+  for (;;) {
+  if (tid == 0) {
+    int x = 0, t = -1;
+    while (tried < kPrefillQueues) {
+      x = (home + tried) & (kPrefillQueues - 1);
+      const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;  // units x, x + 8, ...
+      if (cnt > 0) {
+        t = atomicAdd(a.sched + x, 1);
+        if (t < cnt * tiles) break;
+        t = -1;
+      }
+      ++tried;
+    }
+    sm_ticket[0] = x;
+    sm_ticket[1] = t;
+  }
+  __syncthreads();  // also: every wave is done with the LDS rings of the previous item
+  // (uniform values, kept in scalar registers)
+  const int qx = __builtin_amdgcn_readfirstlane(sm_ticket[0]);
+  const int ticket = __builtin_amdgcn_readfirstlane(sm_ticket[1]);
+  if (ticket < 0) break;  // every queue is empty: the only exit, reached by all workgroups
+  const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
+  const int ti = ticket / qcnt, ui = ticket - ti * qcnt;  // stretch-major: a queue's longest loops first
+  const int u = qx + kPrefillQueues * ui;
+  const int li = u / per_layer, rem = u - li * per_layer;
   const int kvh = rem / hblocks, hb = rem - kvh * hblocks;
-  const int tile = gridDim.y - 1 - blockIdx.y;
+  const int tile = tiles - 1 - ti;
   const int layer = a.layer_begin + li;
   const int window = a.layer_window[layer];
   const int head = kvh * a.group + hb * HPB + (wave % HPB);
-  const int wg_pos0 = a.q_pos0 + tile * (32 * PT);   // first position of the workgroup
-  const int pos_end = a.q_pos0 + a.n;                // one past the last query position
-  const int my_pos0 = wg_pos0 + (wave / HPB) * 32;   // first position of this wave's tile
-  const int row = my_pos0 - a.q_pos0 + n;            // query row in q / out
+  const int wg_pos0 = a.q_pos0 + tile * (kStretch * PT);  // first position of the workgroup
+  const int my_pos0 = wg_pos0 + (wave / HPB) * kStretch;  // first position of this wave's stretch
+  const int row0 = my_pos0 - a.q_pos0 + n;                // query row in q / out
   const int my_pos = my_pos0 + n;
-  const bool row_ok = row < a.n;
 
   const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
   const uint8_t* vplane = kplane + a.geom.plane_bytes;
 
   // Key blocks the workgroup walks: from the first one the window of its first
   // row reaches to the one holding the diagonal of its last valid row. Every
-  // wave walks all of them (blocks outside its own tile's range are masked).
-  const int last_pos = min(wg_pos0 + 32 * PT, pos_end) - 1;
+  // wave walks all of them (blocks outside a tile's range are masked).
+  const int last_pos = min(wg_pos0 + kStretch * PT, pos_end) - 1;
   int kb_lo = 0;
   if (window > 0 && wg_pos0 - window + 1 > 0) kb_lo = (wg_pos0 - window + 1) / kKeysPerBlock;
   const int nblk = last_pos / kKeysPerBlock - kb_lo + 1;
 
   // A K or V block travels HBM/L2 -> LDS without touching registers: every
-  // wave issues 4 of the 16 wave-wide 1 KiB transfers of a block; the data of
-  // lane l lands at the stage offset of the transfer + 16 * l.
-  auto fetch = [&](const uint8_t* plane, uint8_t* ring, int i) {
-    const uint8_t* g = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16;
-    uint8_t* dst = ring + (i % kStages) * kBlockBytes;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int off = (wave + 4 * t) * 1024;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + off),
-                                       (__attribute__((address_space(3))) void*)(dst + off), 16, 0, 0);
-    }
+  // wave issues kXfers of the 16 wave-wide 1 KiB transfers of a block; the data
+  // of lane l lands at the stage offset of the transfer + 16 * l.
+  auto fetch_one = [&](const uint8_t* plane, uint8_t* ring, int i, int t) {
+    const int off = (wave + kWaves * t) * 1024;
+    const uint8_t* g = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16 + off;
+    uint8_t* dst = ring + (i % kStages) * kBlockBytes + off;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
   };
-  // Ring protocol. Iteration i requests K block i+3 and V block i+2: the stage
-  // of K(i+3) held K(i), whose operands went to registers during iteration
-  // i-1; the stage of V(i+2) held V(i-1). At the bottom of iteration i every
-  // wave waits for its share of K(i+2) and V(i+1) (requested one iteration
-  // earlier), so after the barrier iteration i+1 finds V(i+1) and K(i+2)
-  // resident: every transfer has two iterations to land.
+  auto fetch = [&](const uint8_t* plane, uint8_t* ring, int i) {
+#pragma unroll
+    for (int t = 0; t < kXfers; ++t) fetch_one(plane, ring, i, t);
+  };
+  // Ring protocol. Iteration i computes the scores of block i+1 and multiplies
+  // the probabilities of block i-1 into the accumulators, so K runs two blocks
+  // ahead of V: iteration i requests K block i+3 and V block i+1. The stage of
+  // K(i+3) held K(i), read during iteration i-1; the stage of V(i+1) held
+  // V(i-2), also read during iteration i-1. At the bottom of iteration i every
+  // wave waits for its share of K(i+2) and V(i) (requested one iteration
+  // earlier), so after the barrier iteration i+1 finds them resident: every
+  // transfer has a whole iteration to land.
   fetch(kplane, sm_k, 0);
   fetch(vplane, sm_v, 0);
-  if (nblk > 1) { fetch(kplane, sm_k, 1); fetch(vplane, sm_v, 1); }
+  if (nblk > 1) fetch(kplane, sm_k, 1);
   if (nblk > 2) fetch(kplane, sm_k, 2);
 
-  // Q^T operand in this wave's LDS slice: entry (j, lane) with lane = (n, hh)
-  // holds channels 16*j + 8*hh .. +7 of the lane's query. A lane reads back only
-  // what it wrote itself.
-  vec8* const sm_q = sm_q_all + wave * (NJ * 64) + lane;
+  // Q^T operand in registers: slice j of lane (n, hh) holds channels
+  // 16*j + 8*hh .. +7 of the lane's query.
+  vec8 q0[NJ];
   {
-    const elem_t* qrow =
-        reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + (row_ok ? row : 0)) * a.hq + head) * D;
+    const bool ok0 = row0 < a.n;
+    const elem_t* qrow0 =
+        reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + (ok0 ? row0 : 0)) * a.hq + head) * D;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const u4 w = *reinterpret_cast<const u4*>(qrow + 16 * j + 8 * hh);
-      sm_q[j * 64] = bit_cast<vec8>(row_ok ? w : u4{0, 0, 0, 0});
+      const u4 w0 = *reinterpret_cast<const u4*>(qrow0 + 16 * j + 8 * hh);
+      q0[j] = bit_cast<vec8>(ok0 ? w0 : u4{0, 0, 0, 0});
     }
   }
 
-  f16v acc[NDP];
+  f16v acc0[NDP];
 #pragma unroll
   for (int i = 0; i < NDP; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  const float sc = a.scale, softcap = a.softcap;
+    for (int e = 0; e < 16; ++e) acc0[i][e] = 0.f;
+  float m_run0 = -INFINITY, l_run0 = 0.f;
 
-  // LDS offsets of this lane's operands inside a block
-  const int key_row = key_of_row(n);
-  const int k_off = (key_row >> 4) * (16 * D * 2) + (key_row & 15) * 16 + hh * 256;
-  const int v_off = (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
+  // Rare (see kRescaleSlack). The accumulators live in AGPRs (the MFMAs read
+  // and write them there); the pins keep their detour through VGPRs inside
+  // this block.
+  auto rescale = [&](f16v (&acc)[NDP], float alpha) {
+#pragma unroll
+    for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
+#pragma unroll
+    for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
+#pragma unroll
+    for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
+  };
+
+  // Window test in one unsigned comparison: key visible <=> 0 <= pos - key < wlim.
+  const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
+  constexpr int kVAhead = 2;  // channel tiles of V (two operands each) read ahead
+  vec8 kk[kAhead], vv[kVAhead][2];
+  f16v sa, na;                 // scores of the block in the softmax / of the next block
+  vec8 p_prev[NP], p_cur[NP];  // probabilities of the previous block / of this one
+  float bm, alpha, neg_m, lsum;
+
+  // One pipeline step: the vector ALU turns the scores of block i (in sa) into
+  // probabilities while the matrix core multiplies the probabilities of block
+  // i-1 into the accumulators (PREV) and computes the scores of block i+1
+  // (NEXT). The step is cut into one chunk per MFMA; a chunk holds the MFMA,
+  // the LDS read of an operand a few MFMAs ahead and a slice of the softmax,
+  // and the compiler may not move code across chunk borders, so the three
+  // instruction streams stay dealt out evenly. The softmax is a list of 34
+  // pieces: 16 x (soft cap, visibility test, running max of one score), the
+  // exchange of the max between the two lanes of a query (2 pieces, the LDS
+  // crossbar has latency), 16 x (exp2, sum, conversion of one score).
+  // The visibility test is applied to every block, also those in the middle of
+  // the causal triangle: it hides under the MFMAs, and a single variant of the
+  // loop body keeps the accumulators in place.
+  auto step = [&](int i, bool fetch_k, bool fetch_v, auto has_prev, auto has_next) {
+    constexpr bool PREV = decltype(has_prev)::value, NEXT = decltype(has_next)::value;
+    constexpr int GP = PREV ? NDP * NP : 0;  // chunks with a P.V MFMA
+    constexpr int GQ = NEXT ? NJ : 0;        // chunks with a Q.K MFMA
+    constexpr int G = GP + GQ > 0 ? GP + GQ : 1;
+    constexpr int kPieces = 34;
+    const uint8_t* vb = sm_v + ((i + kStages - 1) % kStages) * kBlockBytes + v_off;  // V(i-1)
+    const uint8_t* kb = sm_k + ((i + 1) % kStages) * kBlockBytes + k_off;            // K(i+1)
+    // pos - key of score e is dist0 - (key offset of e inside the block)
+    const int dist0 = my_pos - (kb_lo + i) * kKeysPerBlock - 4 * hh;
+
+    auto piece = [&](auto pc) {
+      constexpr int P = decltype(pc)::value;
+      if constexpr (P < 16) {
+        constexpr int e = P;
+        float x = sa[e];
+        if constexpr (CAP) x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
+        constexpr int koff = 16 * ((e >> 2) & 1) + 8 * (e >> 3) + (e & 3);  // key_of_row(8*(e>>2) + 4*hh + (e&3)) - 4*hh
+        x = (unsigned)(dist0 - koff) < wlim ? x : -INFINITY;
+        sa[e] = x;
+        bm = e == 0 ? x : fmaxf(bm, x);
+      } else if constexpr (P == 16) {
+        lsum = __shfl_xor(bm, 32, 64);  // (lsum is free until the sums start)
+      } else if constexpr (P == 17) {
+        bm = fmaxf(bm, lsum) * c;
+        const float m_new = bm > m_run0 + kRescaleSlack ? bm : m_run0;
+        alpha = (m_run0 == -INFINITY) ? 1.f : fast_exp2(m_run0 - m_new);
+        neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
+        m_run0 = m_new;
+        lsum = 0.f;
+      } else {
+        constexpr int e = P - 18;
+        sa[e] = fast_exp2(fmaf(sa[e], c, neg_m));
+        lsum += sa[e];
+        if constexpr (e & 1) {
+          // probabilities as MFMA operands (bf16: high and low parts, 8
+          // significant bits alone would put ~1e-3 of relative error into P.V)
+#pragma unroll
+          for (int ee = e - 1; ee <= e; ++ee) {
+            const elem_t hi = (elem_t)sa[ee];
+            p_cur[ee >> 3][ee & 7] = hi;
+            if constexpr (DT == kBF16) p_cur[2 + (ee >> 3)][ee & 7] = (elem_t)(sa[ee] - (float)hi);
+          }
+        }
+        // Pins: without them the compiler sinks this arithmetic, whose results
+        // are only needed in the next iteration, out of the chunk.
+        asm volatile("" : "+v"(sa[e]));
+        if constexpr ((e & 7) == 7) {
+          asm volatile("" : "+v"(p_cur[e >> 3]));
+          if constexpr (DT == kBF16) asm volatile("" : "+v"(p_cur[2 + (e >> 3)]));
+        }
+      }
+    };
+
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREV) {
+#pragma unroll
+      for (int dp = 0; dp < kVAhead; ++dp) {
+        vv[dp][0] = *reinterpret_cast<const vec8*>(vb + dp * 2048);
+        vv[dp][1] = *reinterpret_cast<const vec8*>(vb + dp * 2048 + 512);
+      }
+    }
+    if constexpr (NEXT && !PREV) {
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) kk[j] = *reinterpret_cast<const vec8*>(kb + j * 512);
+    }
+    if constexpr (NEXT) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) na[e] = 0.f;
+    }
+    // The transfers of K(i+3) and V(i+1) are requested one at a time, spread
+    // over the step: issued back to back by all four waves they would queue
+    // up in the CU's one vector-memory pipeline and stall the waves in front
+    // of their MFMAs.
+    constexpr int kXferEvery = G >= 2 * kXfers ? G / (2 * kXfers) : 1;
+    static_for<G>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (g % kXferEvery == 0 && g / kXferEvery < 2 * kXfers) {
+        constexpr int t = g / kXferEvery;
+        if (t < kXfers ? fetch_k : fetch_v) {
+          if constexpr (t < kXfers) fetch_one(kplane, sm_k, i + 3, t);
+          else fetch_one(vplane, sm_v, i + 1, t - kXfers);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (g < GP) {
+        constexpr int dp = g / NP, t = g % NP;
+        acc0[dp] = E::mfma(vv[dp % kVAhead][t & 1], p_prev[t], acc0[dp]);
+        if constexpr (t == NP - 1 && dp + kVAhead < NDP) {
+          vv[dp % kVAhead][0] = *reinterpret_cast<const vec8*>(vb + (dp + kVAhead) * 2048);
+          vv[dp % kVAhead][1] = *reinterpret_cast<const vec8*>(vb + (dp + kVAhead) * 2048 + 512);
+        }
+        // the first K operands of the next block, under the last P.V MFMAs
+        if constexpr (NEXT && g >= GP - kAhead)
+          kk[g - (GP - kAhead)] = *reinterpret_cast<const vec8*>(kb + (g - (GP - kAhead)) * 512);
+      } else if constexpr (g < GP + GQ) {
+        constexpr int j = g - GP;
+        na = E::mfma(kk[j % kAhead], q0[j], na);
+        if constexpr (j + kAhead < NJ) kk[j % kAhead] = *reinterpret_cast<const vec8*>(kb + (j + kAhead) * 512);
+      }
+      static_for<kPieces>([&](auto pc) {
+        constexpr int P = decltype(pc)::value;
+        if constexpr (P * G / kPieces == g) piece(pc);
+      });
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    l_run0 = l_run0 * alpha + lsum;
+  };
 
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();  // the first blocks are resident
 
-  // Operand registers: all K slices of the coming block and the first half of
-  // the Q slices are read one phase ahead of their MFMAs.
-  vec8 kop[NJ], qa[NJ / 2], qb[NJ / 2], vop[2 * NDP];
+  constexpr std::true_type yes{};
+  constexpr std::false_type no{};
+  {  // scores of block 0
+    const uint8_t* kb = sm_k + k_off;
 #pragma unroll
-  for (int j = 0; j < NJ; ++j) kop[j] = *reinterpret_cast<const vec8*>(sm_k + k_off + j * 512);
+    for (int j = 0; j < kAhead; ++j) kk[j] = *reinterpret_cast<const vec8*>(kb + j * 512);
 #pragma unroll
-  for (int j = 0; j < NJ / 2; ++j) qa[j] = sm_q[j * 64];
-
-  for (int i = 0; i < nblk; ++i) {
-    const bool fetch_k = i + 3 < nblk, fetch_v = i + 2 < nblk;
-    if (fetch_k) fetch(kplane, sm_k, i + 3);
-    if (fetch_v) fetch(vplane, sm_v, i + 2);
-
-    // ---- S^T = K . Q^T; the second half of the Q slices arrives under the
-    // first eight MFMAs
-#pragma unroll
-    for (int j = 0; j < NJ / 2; ++j) qb[j] = sm_q[(NJ / 2 + j) * 64];
-    f16v s;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s[e] = 0.f;
-#pragma unroll
-    for (int j = 0; j < NJ / 2; ++j) s = E::mfma(kop[j], qa[j], s);
-#pragma unroll
-    for (int j = 0; j < NJ / 2; ++j) s = E::mfma(kop[NJ / 2 + j], qb[j], s);
+    for (int e = 0; e < 16; ++e) sa[e] = 0.f;
+    static_for<NJ>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      sa = E::mfma(kk[j % kAhead], q0[j], sa);
+      if constexpr (j + kAhead < NJ) kk[j % kAhead] = *reinterpret_cast<const vec8*>(kb + (j + kAhead) * 512);
+    });
     __builtin_amdgcn_sched_barrier(0);
-
-    // V operands of this block are requested now and arrive while the softmax runs
-    {
-      const uint8_t* vb = sm_v + (i % kStages) * kBlockBytes + v_off;
+  }
+  auto iteration = [&](int i, auto has_prev, auto has_next) {
+    const bool fetch_k = i + 3 < nblk, fetch_v = i + 1 < nblk;
+    // The accumulators stay in the AGPR half of the register file; scores,
+    // operands and Q^T live in the VGPR half.
 #pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
-        vop[2 * dp] = *reinterpret_cast<const vec8*>(vb + dp * 2048);
-        vop[2 * dp + 1] = *reinterpret_cast<const vec8*>(vb + dp * 2048 + 512);
-      }
-    }
+    for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc0[dp]));
+    step(i, fetch_k, fetch_v, has_prev, has_next);
+    if (__any(alpha != 1.f)) rescale(acc0, alpha);
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < NP; ++t) p_prev[t] = p_cur[t];
+    if constexpr (decltype(has_next)::value) sa = na;
 
-    // ---- online softmax in the exp2 domain; this lane holds 16 keys of query n.
-    // The reference max m_run only moves when some score of the wave exceeds
-    // it by more than kRescaleSlack (2^8 in probability): until then p is
-    // taken against the stale max (p <= 256, harmless in fp32 / fp16 / bf16)
-    // and neither the cross-lane max nor the rescale of the 128 accumulator
-    // registers is needed. m_run is shared by the two lanes of a query.
-    if (softcap > 0.f) {
-      const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) s[e] = cap2 * fast_tanh(s[e] * inv_cap);
-    } else {
-      s *= sc * kLog2e;
-    }
-    const int key0 = (kb_lo + i) * kKeysPerBlock;
-    const bool interior = (key0 + 31 <= my_pos0) && (window <= 0 || my_pos0 + 31 - key0 < window);
-    if (!interior) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = key0 + key_of_row(8 * (e >> 2) + 4 * hh + (e & 3));
-        const bool vis = key <= my_pos && (window <= 0 || my_pos - key < window);
-        s[e] = vis ? s[e] : -INFINITY;
-      }
-    }
-    float bm = s[0];
-#pragma unroll
-    for (int e = 1; e < 16; ++e) bm = fmaxf(bm, s[e]);
-    if (__any(bm > m_run + kRescaleSlack)) {
-      bm = wave_xor_max(bm, 32);
-      const float m_new = fmaxf(m_run, bm);
-      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
-      l_run *= alpha;
-      // The accumulators live in AGPRs (the MFMAs read and write them there);
-      // the two pins keep their detour through VGPRs inside this rare block.
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) acc[dp] *= alpha;
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) asm volatile("" : "+a"(acc[dp]));
-      m_run = m_new;
-    }
-    const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-    float lsum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      s[e] = fast_exp2(s[e] - m_use);
-      lsum += s[e];
-    }
-    l_run += lsum;
-
-    // K operands of the next block (resident since the previous barrier) and
-    // the first half of the Q slices are requested now and arrive during P.V
-    __builtin_amdgcn_sched_barrier(0);
-    if (i + 1 < nblk) {
-      const uint8_t* nx = sm_k + ((i + 1) % kStages) * kBlockBytes + k_off;
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) kop[j] = *reinterpret_cast<const vec8*>(nx + j * 512);
-#pragma unroll
-      for (int j = 0; j < NJ / 2; ++j) qa[j] = sm_q[j * 64];
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- O^T += V^T . P^T
-    if constexpr (DT == kBF16) {
-      // bf16 keeps 8 significant bits; feeding P as hi + lo parts keeps ~16 of
-      // them, otherwise P.V alone carries ~1e-3 of relative error.
-      vec8 p0, p1, q0, q1;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p0[e] = (elem_t)s[e];
-        p1[e] = (elem_t)s[8 + e];
-        q0[e] = (elem_t)(s[e] - (float)p0[e]);
-        q1[e] = (elem_t)(s[8 + e] - (float)p1[e]);
-      }
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
-        acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
-        acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
-        acc[dp] = E::mfma(vop[2 * dp], q0, acc[dp]);
-        acc[dp] = E::mfma(vop[2 * dp + 1], q1, acc[dp]);
-      }
-    } else {
-      vec8 p0, p1;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p0[e] = (elem_t)s[e];
-        p1[e] = (elem_t)s[8 + e];
-      }
-#pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
-        acc[dp] = E::mfma(vop[2 * dp], p0, acc[dp]);
-        acc[dp] = E::mfma(vop[2 * dp + 1], p1, acc[dp]);
-      }
-    }
-
-    // this wave's shares of K(i+2) and V(i+1) have landed; what was requested
-    // in this iteration may still be in flight
-    if (fetch_k) __builtin_amdgcn_s_waitcnt(kWaitVm8);
-    else if (fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm4);
+    // this wave's shares of K(i+2) and V(i) have landed; what was requested in
+    // this iteration may still be in flight
+    if (fetch_k && fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm8);
+    else if (fetch_k || fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm4);
     else __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
+  };
+  if (nblk == 1) {
+    iteration(0, no, no);
+  } else {
+    iteration(0, no, yes);
+    for (int i = 1; i < nblk - 1; ++i) iteration(i, yes, yes);
+    iteration(nblk - 1, yes, no);
+  }
+  {  // the last block's probabilities
+    const uint8_t* vb = sm_v + ((nblk - 1) % kStages) * kBlockBytes + v_off;
+#pragma unroll
+    for (int dp = 0; dp < kVAhead; ++dp) {
+      vv[dp][0] = *reinterpret_cast<const vec8*>(vb + dp * 2048);
+      vv[dp][1] = *reinterpret_cast<const vec8*>(vb + dp * 2048 + 512);
+    }
+    static_for<NDP * NP>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      constexpr int dp = g / NP, t = g % NP;
+      __builtin_amdgcn_sched_barrier(0);
+      acc0[dp] = E::mfma(vv[dp % kVAhead][t & 1], p_prev[t], acc0[dp]);
+      if constexpr (t == NP - 1 && dp + kVAhead < NDP) {
+        vv[dp % kVAhead][0] = *reinterpret_cast<const vec8*>(vb + (dp + kVAhead) * 2048);
+        vv[dp % kVAhead][1] = *reinterpret_cast<const vec8*>(vb + (dp + kVAhead) * 2048 + 512);
+      }
+    });
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- normalise and store: lane (n, hh) holds channels 32*dp + 8*a + 4*hh + b
-  const float l_tot = wave_xor_add(l_run, 32);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (row_ok) {
-    elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
+  auto store = [&](const f16v (&acc)[NDP], float l_run, int row) {
+    const float l_tot = wave_xor_add(l_run, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (row < a.n) {
+      elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
 #pragma unroll
-    for (int dp = 0; dp < NDP; ++dp) {
+      for (int dp = 0; dp < NDP; ++dp) {
 #pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        elem_t o[4];
+        for (int aa = 0; aa < 4; ++aa) {
+          elem_t o[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) o[b] = (elem_t)(acc[dp][4 * aa + b] * inv);
-        *reinterpret_cast<u2*>(orow + 32 * dp + 8 * aa + 4 * hh) = *reinterpret_cast<const u2*>(o);
+          for (int b = 0; b < 4; ++b) o[b] = (elem_t)(acc[dp][4 * aa + b] * inv);
+          *reinterpret_cast<u2*>(orow + 32 * dp + 8 * aa + 4 * hh) = *reinterpret_cast<const u2*>(o);
+        }
       }
     }
+  };
+  store(acc0, l_run0, row0);
+  }  // next work item
+
+  // The last workgroup to get here (all others have drawn their final, failed
+  // tickets) puts the counters back to zero for the next launch.
+  if (tid == 0) {
+    const int done = atomicAdd(a.sched + kPrefillQueues, 1);
+    if (done == (int)gridDim.x - 1)
+      for (int i = 0; i < kPrefillSchedInts; ++i) atomicExch(a.sched + i, 0);
   }
 }
 
-template <int DT, int D, int HPB>
-hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+template <int DT, int D, int HPB, bool CAP>
+hipError_t launch_variant(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill_lds_bytes<D>();
   static bool configured = false;  // more than 64 KiB of LDS has to be requested once per kernel
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB, CAP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
     configured = true;
   }
   // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
-  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB>), grid, dim3(256), kLds, stream, ev0, ev1, 0, a);
+  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB, CAP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
+                        a);
   return hipGetLastError();
+}
+
+template <int DT, int D, int HPB>
+hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  return a.softcap > 0.f ? launch_variant<DT, D, HPB, true>(a, grid, stream, ev0, ev1)
+                         : launch_variant<DT, D, HPB, false>(a, grid, stream, ev0, ev1);
 }
 
 template <int DT, int D>
@@ -348,7 +493,15 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
   const int G = a.group;
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
   const int pt = 4 / hpb;
-  const dim3 grid(a.n_layers * a.geom.hkv * (G / hpb), (a.n + 32 * pt - 1) / (32 * pt), 1);
+  const int items = a.n_layers * a.geom.hkv * (G / hpb) * ((a.n + kStretch * pt - 1) / (kStretch * pt));
+  static int cus = 0;  // one persistent workgroup per CU
+  if (cus == 0) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+  }
+  const dim3 grid(items < cus ? items : cus, 1, 1);
   if (hpb == 4) return launch_hpb<DT, D, 4>(a, grid, stream, ev0, ev1);
   if (hpb == 2) return launch_hpb<DT, D, 2>(a, grid, stream, ev0, ev1);
   return launch_hpb<DT, D, 1>(a, grid, stream, ev0, ev1);
