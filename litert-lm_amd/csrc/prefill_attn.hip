@@ -306,7 +306,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
         }
         // Pins: without them the compiler sinks this arithmetic, whose results
         // are only needed in the next iteration, out of the chunk.
-        asm volatile("" : "+v"(sa[e]));
+        asm volatile("" : "+v"(sa[e]), "+v"(lsum));
         if constexpr ((e & 7) == 7) {
           asm volatile("" : "+v"(p_cur[e >> 3]));
           if constexpr (DT == kBF16) asm volatile("" : "+v"(p_cur[2 + (e >> 3)]));
