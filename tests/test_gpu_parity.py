@@ -403,6 +403,45 @@ def test_c5_int8_full_size_properties():
 
 
 # ------------------------------------------------------------------ error behaviour (no kernel is launched)
+# ------------------------------------------------------------------ golden vectors
+GOLDEN = sorted(__import__("glob").glob(os.path.join(ROOT, "tests", "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+@pytest.mark.parametrize("dt", [A.F32, A.F16, A.BF16])
+def test_golden_vectors(path, dt):
+    """Committed vectors (inputs exactly representable in every dtype, expected
+    output from an independent float64 routine): decode rows go through
+    mi355_attn_decode with several partition counts, chunks through
+    mi355_attn_prefill (MFMA kernel for f16 / bf16, row-wise for f32)."""
+    z = np.load(path)
+    q, k, v, want = z["q"], z["k"], z["v"], z["out"]
+    q_pos0, n, L = int(z["q_pos"][0]), q.shape[0], k.shape[0]
+    window, scale, softcap = int(z["window"]), float(z["scale"]), float(z["softcap"])
+    hq, hkv = q.shape[1], k.shape[1]
+    assert q_pos0 + n == L
+    with make(1, hq, hkv, L, 1, dt, layer_window=[window], scale=scale, softcap=softcap) as at:
+        kd, kr = dev(k, dt)
+        vd, vr = dev(v, dt)
+        assert np.array_equal(kr, k) and np.array_equal(vr, v)  # nothing is lost entering the cache
+        at.kv_append(0, 0, 0, kd, vd)
+        qd, qr = dev(q, dt)
+        assert np.array_equal(qr, q)
+        out = torch.empty_like(qd)
+        if n == 1:
+            for splits in (0, 1, 2):
+                at.decode(0, [L], qd, out, num_splits=splits)
+                torch.cuda.synchronize()
+                err = err_of(out.float().cpu().numpy(), want, dt)
+                assert err < TOL[dt], (os.path.basename(path), dt, splits, err)
+        else:
+            at.prefill(0, 0, q_pos0, n, qd, out)
+            torch.cuda.synchronize()
+            err = err_of(out.float().cpu().numpy(), want, dt)
+            assert err < TOL[dt], (os.path.basename(path), dt, err)
+        say(f"golden {os.path.basename(path)} dt={dt}: rel_err={err:.3e}")
+
+
 def test_error_codes():
     with pytest.raises(A.AttnError) as e:
         A.Attn(1, 3, 2, D, 16, 1, A.F16, A.F16)
