@@ -214,6 +214,35 @@ def gemm_probe(torch, n=8192, reps=20):
     return 2 * n ** 3 / sec / 1e12
 
 
+def bench_sampler(S, torch, steps, warmup, batch=64, vocab=262144, k=64, p=0.95, rotation=8):
+    """Token sampling right after the attention path: [batch, vocab] float32 logits in HBM ->
+    one id per row (top-k 64, top-p 0.95). Rotates over `rotation` logits tensors (512 MiB)."""
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device="cuda:0").manual_seed(0xC0FFEE + 7)
+    logits = [torch.randn((batch, vocab), generator=g, device="cuda:0") * 3.0 for _ in range(rotation)]
+    ids = torch.zeros((batch,), dtype=torch.int32, device="cuda:0")
+    with S.Sampler(k, p, 1.0, batch, 1, vocab, stream=stream) as s:
+        def step(i):
+            s.sample_to_id_and_score_buffer(logits[i % rotation], ids)
+        sec = time_steps(torch, step, steps, warmup)
+        s.set_timing(True)
+        total = 0.0
+        for i in range(min(steps, 30)):
+            step(i)
+            total += s.last_kernel_ms()
+        s.set_timing(False)
+        kms = total / min(steps, 30)
+    with S.Sampler(k, p, 1.0, 1, 1, vocab, stream=stream) as s1:
+        one = logits[0][:1].contiguous()
+        id1 = torch.zeros((1,), dtype=torch.int32, device="cuda:0")
+        lat = time_steps(torch, lambda i: s1.sample_to_id_and_score_buffer(one, id1), 200, 20)
+    nbytes = batch * vocab * 4
+    return {"workload": f"sampling: {batch} rows x {vocab} float32 logits, top-k {k}, top-p {p}, one launch",
+            "ms_per_step": sec * 1e3, "kernel_ms": kms, "bytes": nbytes, "GBps": nbytes / sec / 1e9,
+            "kernel_GBps": nbytes / (kms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "tokens_per_s": batch / sec, "single_row_latency_us": lat * 1e6}
+
+
 def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=12.0):
     """C restatement of the reference CPU op order (fp32, OpenMP) on the same
     30-layer decode sweep, repeated until about `budget_s` seconds are spent."""
@@ -341,6 +370,10 @@ def main():
         log(f"[bench] {c1['workload']}: {c1['ms_per_step']*1e3:.1f} us/step")
         extras.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in c1.items()})
         result["other_decode_configs"] = extras
+        smp = bench_sampler(load_package().sampler, torch, max(20, args.steps // 4), max(5, args.warmup // 4))
+        log(f"[bench] {smp['workload']}: {smp['ms_per_step']*1e3:.1f} us/step, kernel {smp['kernel_GBps']:.0f} GB/s, "
+            f"one row {smp['single_row_latency_us']:.1f} us")
+        result["sampler"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in smp.items()}
 
     if not args.no_cpu:
         cpu = cpu_baseline_c3(dec["layers"], 4096, dec["step_bytes"])

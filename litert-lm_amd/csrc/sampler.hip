@@ -1,0 +1,700 @@
+// Token sampling on the device (gfx950): top-k -> softmax with temperature ->
+// top-p nucleus -> one draw.
+//
+// Replaces the reference's CPU arithmetic
+//   TopKIndicies       runtime/components/sampling_cpu_util.cc:21-64
+//   Softmax            runtime/components/sampling_cpu_util.cc:66-134
+//   TopKTopPSampling   runtime/components/sampling_cpu_util.cc:136-233
+// behind the C ABI shape of its GPU sampler plugin
+// (runtime/components/sampler_factory.cc:34-46).
+//
+// Two launches per call. select_kernel: a row of ~262k logits is cut into up to
+// 16 segments, one workgroup of 1024 threads each, so that one row already
+// spreads over 16 CUs. A workgroup finds the k largest of its segment in two
+// passes over it (the second one an L2 hit): every thread keeps the maximum of
+// the logits it reads; the k-th largest of those 1024 maxima is a lower bound of
+// the segment's k-th largest logit, so the second pass only has to collect what
+// reaches it - a few hundred candidates, which a bitonic sort in LDS orders
+// (descending value, equal values by ascending index). Segments for which that
+// bound is too weak (more than 2048 candidates: long runs of equal values) fall
+// back to a radix descent on an order-preserving 32-bit key with LDS histograms
+// (12 + 12 + 8 bits); exact ties at the k-th value are then taken in ascending
+// index order. finish_kernel: one workgroup per row merges the segments'
+// candidates by another sort and one thread walks the k winners in the
+// reference's op order.
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+#include <float.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "../../include/mi355_sampler.h"
+
+namespace {
+
+constexpr int kThreads = 1024;
+constexpr int kWavesPerWg = kThreads / 64;
+constexpr int kPerIter = kThreads * 4;  // logits per pass iteration: 4 consecutive ones per thread
+constexpr int kUnroll = 4;              // iterations whose loads are in flight together
+constexpr int kBins = 4096;
+constexpr int kCap = 2048;              // candidates of one segment that fit in LDS for the sort
+constexpr int kMaxK = MI355_SAMPLER_MAX_K;
+constexpr int kMaxSegments = 16;
+constexpr int kMergeCap = kMaxSegments * kMaxK;  // 4096 candidates of one row in finish_kernel
+constexpr int kResident = 16;           // logits per thread that stay in registers between the passes
+constexpr int kSegmentMin = kThreads * kResident;  // a segment is this long unless the row needs more than kMaxSegments
+
+typedef unsigned long long u64;
+
+struct SamplerArgs {
+  const float* logits;    // [batch][vocab]
+  const float* uniforms;  // [batch] or null: Philox draws
+  int32_t* ids;           // [batch] or null
+  float* scores;          // [batch] or null
+  int32_t* topk_idx;      // [batch][k] or null
+  float* topk_prob;       // [batch][k] or null
+  u64* workspace;         // [batch][segments][k] candidates, (key << 32) | ~index
+  int32_t vocab, k, segments, seg_len;
+  float p, temperature;
+  uint32_t seed;
+  uint64_t call_index;
+};
+
+// Larger float <=> larger key; -0 and +0 share a key; NaN sorts below everything.
+__device__ __forceinline__ uint32_t key_of(float x) {
+  if (x != x) return 0u;
+  uint32_t u = __float_as_uint(x == 0.f ? 0.f : x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float logit_of(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+// Candidate word: descending order of the word = descending key, then ascending index.
+__device__ __forceinline__ u64 pack(uint32_t key, int index) { return ((u64)key << 32) | (uint32_t)~(uint32_t)index; }
+__device__ __forceinline__ int index_of(u64 c) { return (int)~(uint32_t)c; }
+
+__device__ __forceinline__ void philox_round(uint32_t (&c)[4], uint32_t (&k)[2]) {
+  const uint32_t lo0 = 0xD2511F53u * c[0], hi0 = __umulhi(0xD2511F53u, c[0]);
+  const uint32_t lo1 = 0xCD9E8D57u * c[2], hi1 = __umulhi(0xCD9E8D57u, c[2]);
+  const uint32_t n0 = hi1 ^ c[1] ^ k[0], n2 = hi0 ^ c[3] ^ k[1];
+  c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
+  k[0] += 0x9E3779B9u; k[1] += 0xBB67AE85u;
+}
+// Philox4x32-10 (Salmon et al., SC'11); the first output word.
+__device__ __forceinline__ uint32_t philox_first_word(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                      uint32_t k1) {
+  uint32_t c[4] = {c0, c1, c2, c3}, k[2] = {k0, k1};
+#pragma unroll
+  for (int r = 0; r < 10; ++r) philox_round(c, k);
+  return c[0];
+}
+
+// One pass over a segment: f(key, local index) for every logit, 4 consecutive
+// ones per thread and iteration (so that waves, lanes and elements run in
+// ascending index order), the loads of kUnroll iterations in flight together.
+template <class F>
+__device__ __forceinline__ void for_each_key(const float* seg, int len, bool vec_ok, int tid, F&& f) {
+  int base = tid * 4;
+  if (vec_ok) {
+    for (; base + (kUnroll - 1) * kPerIter + 3 < len; base += kUnroll * kPerIter) {
+      float4 x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) x[u] = *reinterpret_cast<const float4*>(seg + base + u * kPerIter);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int i = base + u * kPerIter;
+        f(key_of(x[u].x), i); f(key_of(x[u].y), i + 1); f(key_of(x[u].z), i + 2); f(key_of(x[u].w), i + 3);
+      }
+    }
+    for (; base + 3 < len; base += kPerIter) {
+      const float4 x = *reinterpret_cast<const float4*>(seg + base);
+      f(key_of(x.x), base); f(key_of(x.y), base + 1); f(key_of(x.z), base + 2); f(key_of(x.w), base + 3);
+    }
+  }
+  for (; base < len; base += kPerIter)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (base + j < len) f(key_of(seg[base + j]), base + j);
+}
+
+// The bin, counted from the top, in which the cumulative count of hist[0..nbins)
+// reaches `need` (1 <= need <= total): found = {bin, count above it, count in it}.
+// Thread t owns bins 4t .. 4t+3; suffix sums over the threads above it. Ends
+// with a barrier; found[] is valid for every thread afterwards.
+__device__ __forceinline__ void find_bin(const uint32_t* hist, int nbins, uint32_t need, uint32_t* wave_sum,
+                                         uint32_t* found, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  uint32_t h[4], s = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) { h[j] = 4 * tid + j < nbins ? hist[4 * tid + j] : 0u; s += h[j]; }
+  uint32_t incl = s;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t v = __shfl_down(incl, off, 64);
+    if (lane + off < 64) incl += v;
+  }
+  if (lane == 0) wave_sum[wave] = incl;
+  __syncthreads();
+  uint32_t cum = incl - s;
+  for (int w = wave + 1; w < kWavesPerWg; ++w) cum += wave_sum[w];
+#pragma unroll
+  for (int j = 3; j >= 0; --j) {
+    if (cum < need && cum + h[j] >= need) { found[0] = 4 * tid + j; found[1] = cum; found[2] = h[j]; }
+    cum += h[j];
+  }
+  __syncthreads();
+}
+
+// Maximum over the wave, in every lane, by DPP row shifts and row broadcasts
+// (no LDS round trips). 0 is the identity.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#define MI355_DPP_MAX(ctrl, row_mask) \
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, row_mask, 0xf, false))
+  MI355_DPP_MAX(0x111, 0xf);  // row_shr:1
+  MI355_DPP_MAX(0x112, 0xf);  // row_shr:2
+  MI355_DPP_MAX(0x114, 0xf);  // row_shr:4
+  MI355_DPP_MAX(0x118, 0xf);  // row_shr:8   -> lane 15 of each row of 16 holds the row's maximum
+  MI355_DPP_MAX(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+  MI355_DPP_MAX(0x143, 0xc);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave's maximum
+#undef MI355_DPP_MAX
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// A lower bound that at least k of the values v (one per thread, 0 = none) reach:
+// every wave reports the j-th largest of its 64 values, j = ceil(k / 16); at
+// least 16 j >= k values reach the smallest of those 16 numbers. One barrier.
+__device__ __forceinline__ uint32_t lower_bound_of_kth(uint32_t v, int k, uint32_t* wave_val, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  const int j_th = (k + kWavesPerWg - 1) / kWavesPerWg;
+  uint32_t m = 0;
+  for (int r = 0; r < j_th; ++r) {
+    m = wave_max_u32(v);
+    const u64 holders = __ballot(v == m);
+    if (lane == __ffsll((long long)holders) - 1) v = 0;  // drop one holder of the maximum
+  }
+  if (lane == 0) wave_val[wave] = m;
+  __syncthreads();
+  uint32_t tau = wave_val[0];
+  for (int w = 1; w < kWavesPerWg; ++w) tau = min(tau, wave_val[w]);
+  return tau;
+}
+
+// top[r] = the candidate of rank r (number of larger candidates; the words are
+// distinct) for r < k, by counting instead of sorting: 256 candidates at a
+// time, the comparisons of each split over 4 threads.
+__device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, int k, uint32_t* rank_sm, int tid) {
+  const int slot = tid & 255, part = tid >> 8;
+  const int span = (n + 3) / 4, j0 = part * span, j1 = min(n, j0 + span);
+  for (int blk = 0; blk < n; blk += 256) {
+    if (tid < 256) rank_sm[tid] = 0;
+    __syncthreads();
+    if (blk + slot < n) {
+      const u64 c = cand[blk + slot];
+      uint32_t cnt = 0;
+      for (int j = j0; j < j1; j += 8) {  // eight independent LDS reads in flight
+        u64 x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = j + u < j1 ? cand[j + u] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) cnt += x[u] > c ? 1u : 0u;
+      }
+      if (cnt) atomicAdd(&rank_sm[slot], cnt);
+    }
+    __syncthreads();
+    if (tid < 256 && blk + tid < n && rank_sm[tid] < (uint32_t)k) top[rank_sm[tid]] = cand[blk + tid];
+    __syncthreads();
+  }
+}
+
+// The k largest logits of one segment of one row, sorted, into the workspace.
+__global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
+  __shared__ uint32_t hist[kBins];
+  __shared__ u64 cand[kCap];
+  __shared__ u64 top[kMaxK];
+  __shared__ uint32_t rank_sm[256];
+  __shared__ uint32_t wave_sum[kWavesPerWg];
+  __shared__ uint32_t found[3];  // bin, count above it, count in it
+  __shared__ uint32_t n_cand, n_ties;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = blockIdx.y, sgm = blockIdx.x;
+  const int index0 = sgm * a.seg_len;                 // first vocabulary index of the segment
+  const int len = min(a.seg_len, a.vocab - index0);   // > 0 by construction of the grid
+  const int k = min(a.k, len);
+  const float* seg = a.logits + (size_t)b * a.vocab + index0;
+  const bool vec_ok = (a.vocab % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
+  u64* out = a.workspace + ((size_t)b * a.segments + sgm) * a.k;
+
+  // A segment of up to 16 logits per thread is read from memory once: its keys
+  // stay in registers for all later passes (same index layout as for_each_key).
+  const bool resident = len <= kThreads * kResident;
+  uint32_t kreg[kResident];
+  if (resident) {
+#pragma unroll
+    for (int u = 0; u < kResident / 4; ++u) {
+      const int base = u * kPerIter + tid * 4;
+      if (vec_ok && base + 3 < len) {
+        const float4 x = *reinterpret_cast<const float4*>(seg + base);
+        kreg[4 * u] = key_of(x.x); kreg[4 * u + 1] = key_of(x.y); kreg[4 * u + 2] = key_of(x.z); kreg[4 * u + 3] = key_of(x.w);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) kreg[4 * u + j] = base + j < len ? key_of(seg[base + j]) : 0u;
+      }
+    }
+  }
+  auto each = [&](auto&& f) {
+    if (resident) {
+#pragma unroll
+      for (int u = 0; u < kResident / 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = u * kPerIter + tid * 4 + j;
+          if (i < len) f(kreg[4 * u + j], i);
+        }
+    } else {
+      for_each_key(seg, len, vec_ok, tid, f);
+    }
+  };
+
+  if (k == 1) {
+    // the first maximum (std::max_element), one pass
+    u64 best = 0;
+    each([&](uint32_t key, int i) { best = max(best, pack(key, index0 + i)); });
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) best = max(best, (u64)__shfl_xor((long long)best, off, 64));
+    if (lane == 0) cand[wave] = best;
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 1; w < kWavesPerWg; ++w) best = max(best, cand[w]);
+      out[0] = best;
+    }
+    for (int i = 1 + tid; i < a.k; i += kThreads) out[i] = 0;
+    return;
+  }
+
+  // ---- a threshold from the per-thread maxima, then everything that reaches it
+  {
+    uint32_t tmax = 0;
+    each([&](uint32_t key, int) { tmax = max(tmax, key); });
+    if (tid == 0) n_cand = 0;
+    const uint32_t tau = lower_bound_of_kth(tmax, k, wave_sum, tid);  // (barrier inside)
+    uint32_t mine = 0;
+    each([&](uint32_t key, int) { mine += key >= tau ? 1u : 0u; });
+    uint32_t pos = mine ? atomicAdd(&n_cand, mine) : 0u;
+    each([&](uint32_t key, int i) {
+      if (key >= tau) {
+        if (pos < (uint32_t)kCap) cand[pos] = pack(key, index0 + i);
+        ++pos;
+      }
+    });
+    __syncthreads();
+  }
+  const bool fast_ok = n_cand <= (uint32_t)kCap;
+  __syncthreads();
+
+  if (!fast_ok) {
+    // ---- radix descent: (mask, val) = the key prefix of the k-th largest value so far
+    uint32_t mask = 0, val = 0, need = (uint32_t)k;
+    bool exact_ties = false;
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 20 : (level == 1 ? 8 : 0);
+      const int nbins = level == 2 ? 256 : kBins;
+      for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
+      __syncthreads();
+      each([&](uint32_t key, int) {
+        if ((key & mask) == val) atomicAdd(&hist[(key >> shift) & (nbins - 1)], 1u);
+      });
+      __syncthreads();
+      find_bin(hist, nbins, need, wave_sum, found, tid);
+      val |= found[0] << shift;
+      mask |= (uint32_t)(nbins - 1) << shift;
+      need -= found[1];
+      const uint32_t in_bin = found[2];
+      if (in_bin + ((uint32_t)k - need) <= (uint32_t)kCap) break;
+      exact_ties = level == 2;  // the whole key is fixed and still too many: equal values
+      __syncthreads();          // found[] is rewritten by the next level
+    }
+
+    // ---- collection: everything above the prefix, and the prefix bin itself
+    // (of exact ties only the `need` lowest indices)
+    if (tid == 0) { n_cand = 0; n_ties = 0; }
+    __syncthreads();
+    if (!exact_ties) {
+      each([&](uint32_t key, int i) {
+        if ((key & mask) >= val) cand[atomicAdd(&n_cand, 1u)] = pack(key, index0 + i);
+      });
+    } else {
+      // every iteration in step, so that ties are ranked in index order: waves,
+      // lanes and a thread's four elements are laid out ascending
+      for (int base0 = 0; base0 < len; base0 += kPerIter) {
+        const int base = base0 + tid * 4;
+        uint32_t key[4];
+        int mine = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          key[j] = base + j < len ? key_of(seg[base + j]) : 0u;
+          if (base + j < len && key[j] > val) cand[atomicAdd(&n_cand, 1u)] = pack(key[j], index0 + base + j);
+          if (base + j < len && key[j] == val) ++mine;
+        }
+        uint32_t incl = (uint32_t)mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const uint32_t v = __shfl_up(incl, off, 64);
+          if (lane >= off) incl += v;
+        }
+        if (lane == 63) wave_sum[wave] = incl;
+        __syncthreads();
+        uint32_t rank = n_ties + incl - (uint32_t)mine, total = 0;
+        for (int w = 0; w < kWavesPerWg; ++w) { if (w < wave) rank += wave_sum[w]; total += wave_sum[w]; }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (base + j < len && key[j] == val) {
+            if (rank < need) cand[atomicAdd(&n_cand, 1u)] = pack(key[j], index0 + base + j);
+            ++rank;
+          }
+        __syncthreads();
+        if (tid == 0) n_ties += total;
+        __syncthreads();
+      }
+    }
+    __syncthreads();
+  }
+  const int n = (int)n_cand;  // k <= n <= kCap
+  rank_select(cand, n, top, k, rank_sm, tid);
+  for (int i = tid; i < a.k; i += kThreads) out[i] = i < k ? top[i] : 0;
+}
+
+// Merges the segments' candidates of one row and draws (sampling_cpu_util.cc:98-131, 189-230).
+__global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
+  __shared__ u64 surv[kMergeCap];  // the segments' candidates that reach the threshold
+  __shared__ u64 cand[kMaxK];      // the row's k winners, descending
+  __shared__ float e_sm[kMaxK];
+  __shared__ uint32_t rank_sm[256];
+  __shared__ uint32_t wave_val[kWavesPerWg];
+  __shared__ uint32_t n_surv;
+  __shared__ float inv_sm;
+  __shared__ double cum_sm[kMaxK];
+  __shared__ int first_reach, first_hit;
+  const int tid = threadIdx.x, b = blockIdx.x;
+  const int k = min(a.k, a.vocab);
+  const int n = a.segments * a.k;  // <= kMergeCap: up to 4 words per thread; zero words are empty slots
+  const u64* in = a.workspace + (size_t)b * n;
+  u64 w[4];
+  uint32_t wmax = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    w[j] = tid + j * kThreads < n ? in[tid + j * kThreads] : 0;
+    wmax = max(wmax, (uint32_t)(w[j] >> 32));
+  }
+  if (tid == 0) { n_surv = 0; first_reach = k - 1; first_hit = kMaxK; }
+  // same scheme as in select_kernel: a lower bound of the k-th largest key, the
+  // words that reach it, their ranks by counting
+  const uint32_t tau = lower_bound_of_kth(wmax, k, wave_val, tid);  // (barrier inside)
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) mine += (w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau) ? 1u : 0u;
+  uint32_t pos = mine ? atomicAdd(&n_surv, mine) : 0u;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau) surv[pos++] = w[j];
+  __syncthreads();
+  rank_select(surv, (int)n_surv, cand, k, rank_sm, tid);
+
+  if (k == 1) {
+    if (tid == 0) {
+      const int idx = index_of(cand[0]);
+      if (a.ids) a.ids[b] = idx;
+      if (a.scores) a.scores[b] = 0.f;  // log(1)
+      if (a.topk_idx) a.topk_idx[b] = idx;
+      if (a.topk_prob) a.topk_prob[b] = 1.f;
+    }
+    return;
+  }
+  // ---- the k winners in the reference's op order (sampling_cpu_util.cc:98-131, 189-230)
+  const float m = logit_of((uint32_t)(cand[0] >> 32));
+  const float t_soft = fmaxf(a.temperature, FLT_EPSILON);
+  if (tid < k) e_sm[tid] = expf((logit_of((uint32_t)(cand[tid] >> 32)) - m) / t_soft);
+  __syncthreads();
+  if (tid == 0) {
+    // sequential float32 sum, as the reference; the LDS reads run ahead of the adds
+    float sum = 0.f;
+    for (int i = 0; i < k; i += 8) {
+      float x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) x[u] = i + u < k ? e_sm[i + u] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum += x[u];
+    }
+    inv_sm = sum <= FLT_EPSILON ? -1.f : (isinf(sum) ? -2.f : 1.f / sum);
+  }
+  __syncthreads();
+  if (tid < k) {
+    const float inv = inv_sm;
+    e_sm[tid] = inv == -1.f ? 1.f / (float)k : (inv == -2.f ? (tid == 0 ? 1.f : 0.f) : e_sm[tid] * inv);
+  }
+  __syncthreads();
+  // Cumulative probabilities in float64, every thread summing its own prefix in
+  // the reference's order; the nucleus ends at the first one that reaches p, the
+  // draw picks the first one that covers it (sampling_cpu_util.cc:189-230).
+  if (tid < k) {
+    double c = 0.0;
+    for (int i = 0; i <= tid; i += 8) {
+      float x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) x[u] = i + u <= tid ? e_sm[i + u] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c += (double)x[u];
+    }
+    cum_sm[tid] = c;
+    if (c >= (double)a.p) atomicMin(&first_reach, tid);
+  }
+  __syncthreads();
+  const int nucleus = first_reach + 1;  // first_reach starts at k - 1: never reached = all k candidates
+  const double mass = cum_sm[first_reach];
+  float u01;
+  if (a.uniforms) u01 = a.uniforms[b];
+  else u01 = (float)(philox_first_word((uint32_t)b, (uint32_t)a.call_index, (uint32_t)(a.call_index >> 32), 0u, a.seed,
+                                       0x4D493335u) >> 8) * (1.f / 16777216.f);
+  const double draw = (double)u01 * mass;
+  if (tid < nucleus && draw <= cum_sm[tid]) atomicMin(&first_hit, tid);
+  __syncthreads();
+  if (tid == 0) {
+    const int chosen = mass > DBL_EPSILON ? min(first_hit, nucleus - 1) : 0;
+    if (a.ids) a.ids[b] = index_of(cand[chosen]);
+    if (a.scores) a.scores[b] = logf(expf((logit_of((uint32_t)(cand[chosen] >> 32)) - m) / a.temperature));
+  }
+  __syncthreads();
+  if (tid < k) {
+    if (a.topk_idx) a.topk_idx[(size_t)b * k + tid] = index_of(cand[tid]);
+    if (a.topk_prob) a.topk_prob[(size_t)b * k + tid] = e_sm[tid];
+  }
+}
+
+int fail(char** error_msg, int code, const char* fmt, ...) {
+  if (error_msg) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    *error_msg = strdup(buf);
+  }
+  return code;
+}
+
+#define HIP_OR_RETURN(expr)                                                                          \
+  do {                                                                                               \
+    hipError_t e_ = (expr);                                                                          \
+    if (e_ != hipSuccess)                                                                            \
+      return fail(error_msg, e_ == hipErrorOutOfMemory ? MI355_SAMPLER_RESOURCE_EXHAUSTED            \
+                                                        : MI355_SAMPLER_INTERNAL,                    \
+                  "%s: %s", #expr, hipGetErrorString(e_));                                           \
+  } while (0)
+
+}  // namespace
+
+struct mi355_sampler {
+  mi355_sampler_config cfg{};
+  int k = 1;
+  float p = 1.f;
+  hipStream_t stream = nullptr;
+  bool owns_stream = false;
+  uint64_t calls = 0;
+  bool timing = false, timed = false;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  // host_io staging
+  float* d_logits = nullptr;
+  float* d_uniforms = nullptr;
+  int32_t* d_ids = nullptr;
+  float* d_scores = nullptr;
+  int32_t* d_topk_idx = nullptr;
+  float* d_topk_prob = nullptr;
+  // candidates of the segments, [batch][segments][k]
+  unsigned long long* d_workspace = nullptr;
+  int segments = 1, seg_len = 0;
+};
+
+namespace {
+
+int run(mi355_sampler* h, const float* logits, const float* uniforms, int32_t* ids, float* scores, int32_t* topk_idx,
+        float* topk_prob, bool counts_as_draw, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null sampler");
+  if (!logits) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null logits");
+  HIP_OR_RETURN(hipSetDevice(h->cfg.device));
+  const size_t B = h->cfg.batch_size, V = h->cfg.vocab_size, K = std::min<size_t>(h->k, V);
+  SamplerArgs a{};
+  if (h->cfg.host_io) {
+    HIP_OR_RETURN(hipMemcpyAsync(h->d_logits, logits, B * V * sizeof(float), hipMemcpyHostToDevice, h->stream));
+    if (uniforms)
+      HIP_OR_RETURN(hipMemcpyAsync(h->d_uniforms, uniforms, B * sizeof(float), hipMemcpyHostToDevice, h->stream));
+    a.logits = h->d_logits;
+    a.uniforms = uniforms ? h->d_uniforms : nullptr;
+    a.ids = ids ? h->d_ids : nullptr;
+    a.scores = scores ? h->d_scores : nullptr;
+    a.topk_idx = topk_idx ? h->d_topk_idx : nullptr;
+    a.topk_prob = topk_prob ? h->d_topk_prob : nullptr;
+  } else {
+    a.logits = logits; a.uniforms = uniforms; a.ids = ids; a.scores = scores;
+    a.topk_idx = topk_idx; a.topk_prob = topk_prob;
+  }
+  a.vocab = (int32_t)V;
+  a.k = h->k;
+  a.p = h->p;
+  a.temperature = h->cfg.temperature;
+  a.seed = (uint32_t)h->cfg.seed;
+  a.call_index = h->calls;
+  if (counts_as_draw) ++h->calls;
+  a.workspace = h->d_workspace;
+  a.segments = h->segments;
+  a.seg_len = h->seg_len;
+  // ev0 / ev1 ride on the dispatches: begin of the first kernel, end of the second
+  hipExtLaunchKernelGGL(select_kernel, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
+                        h->timing ? h->ev0 : nullptr, nullptr, 0, a);
+  HIP_OR_RETURN(hipGetLastError());
+  hipExtLaunchKernelGGL(finish_kernel, dim3((unsigned)B), dim3(kThreads), 0, h->stream, nullptr,
+                        h->timing ? h->ev1 : nullptr, 0, a);
+  HIP_OR_RETURN(hipGetLastError());
+  h->timed = h->timing;
+  if (h->cfg.host_io) {
+    if (ids) HIP_OR_RETURN(hipMemcpyAsync(ids, h->d_ids, B * sizeof(int32_t), hipMemcpyDeviceToHost, h->stream));
+    if (scores) HIP_OR_RETURN(hipMemcpyAsync(scores, h->d_scores, B * sizeof(float), hipMemcpyDeviceToHost, h->stream));
+    if (topk_idx)
+      HIP_OR_RETURN(hipMemcpyAsync(topk_idx, h->d_topk_idx, B * K * sizeof(int32_t), hipMemcpyDeviceToHost, h->stream));
+    if (topk_prob)
+      HIP_OR_RETURN(hipMemcpyAsync(topk_prob, h->d_topk_prob, B * K * sizeof(float), hipMemcpyDeviceToHost, h->stream));
+    HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  }
+  return MI355_SAMPLER_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_sampler_create(const mi355_sampler_config* c, mi355_sampler** out, char** error_msg) {
+  if (!c || !out) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null config or output pointer");
+  *out = nullptr;
+  if (c->struct_size != sizeof(mi355_sampler_config))
+    return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "mi355_sampler_config.struct_size %u, expected %zu",
+                c->struct_size, sizeof(mi355_sampler_config));
+  int k = c->k;
+  float p = c->p;
+  switch (c->type) {
+    case MI355_SAMPLER_GREEDY: k = 1; p = 1.f; break;
+    case MI355_SAMPLER_TOP_K: p = 1.f; break;
+    case MI355_SAMPLER_TOP_P:
+    case MI355_SAMPLER_TYPE_UNSPECIFIED: break;
+    default: return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "unknown sampler type %d", c->type);
+  }
+  // messages of TopPSampler::Create (top_p_cpu_sampler.cc:42-55)
+  if (k <= 0) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "k must be positive.");
+  if (!(p >= 0.0f && p <= 1.0f)) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "p must be in [0, 1].");
+  if (c->batch_size <= 0) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "batch_size must be positive.");
+  if (!(c->temperature > 0.0f))
+    return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "Temperature must be positive, but got %g", c->temperature);
+  if (c->vocab_size <= 0) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "vocab_size must be positive.");
+  if (std::min(k, c->vocab_size) > kMaxK)
+    return fail(error_msg, MI355_SAMPLER_UNIMPLEMENTED, "k = %d: at most %d candidates are supported", k, kMaxK);
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || c->device < 0 || c->device >= ndev)
+    return fail(error_msg, MI355_SAMPLER_UNAVAILABLE, "no usable HIP device %d", c->device);
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, c->device) != hipSuccess || strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(error_msg, MI355_SAMPLER_UNAVAILABLE, "device %d is not gfx950", c->device);
+  HIP_OR_RETURN(hipSetDevice(c->device));
+  mi355_sampler* h = new mi355_sampler();
+  h->cfg = *c;
+  h->k = k;
+  h->p = p;
+  auto bail = [&](int code, const char* what, hipError_t e) {
+    mi355_sampler_destroy(h);
+    return fail(error_msg, code, "%s: %s", what, hipGetErrorString(e));
+  };
+  hipError_t e;
+  if (c->own_stream) {
+    if ((e = hipStreamCreate(&h->stream)) != hipSuccess) return bail(MI355_SAMPLER_INTERNAL, "hipStreamCreate", e);
+    h->owns_stream = true;
+  } else {
+    h->stream = static_cast<hipStream_t>(c->stream);
+  }
+  if ((e = hipEventCreate(&h->ev0)) != hipSuccess || (e = hipEventCreate(&h->ev1)) != hipSuccess)
+    return bail(MI355_SAMPLER_INTERNAL, "hipEventCreate", e);
+  // segments of kSegmentMin logits or less (a multiple of 4), unless that would take more than kMaxSegments
+  h->segments = std::max(1, std::min(kMaxSegments, (c->vocab_size + kSegmentMin - 1) / kSegmentMin));
+  h->seg_len = ((c->vocab_size + h->segments - 1) / h->segments + 3) / 4 * 4;
+  h->segments = (c->vocab_size + h->seg_len - 1) / h->seg_len;
+  if ((e = hipMalloc(&h->d_workspace, sizeof(unsigned long long) * c->batch_size * h->segments * k)) != hipSuccess)
+    return bail(MI355_SAMPLER_RESOURCE_EXHAUSTED, "candidate workspace", e);
+  if (c->host_io) {
+    const size_t B = c->batch_size, V = c->vocab_size, K = std::min<size_t>(k, V);
+    if ((e = hipMalloc(&h->d_logits, B * V * sizeof(float))) != hipSuccess ||
+        (e = hipMalloc(&h->d_uniforms, B * sizeof(float))) != hipSuccess ||
+        (e = hipMalloc(&h->d_ids, B * sizeof(int32_t))) != hipSuccess ||
+        (e = hipMalloc(&h->d_scores, B * sizeof(float))) != hipSuccess ||
+        (e = hipMalloc(&h->d_topk_idx, B * K * sizeof(int32_t))) != hipSuccess ||
+        (e = hipMalloc(&h->d_topk_prob, B * K * sizeof(float))) != hipSuccess)
+      return bail(MI355_SAMPLER_RESOURCE_EXHAUSTED, "staging buffers", e);
+  }
+  *out = h;
+  return MI355_SAMPLER_OK;
+}
+
+void mi355_sampler_destroy(mi355_sampler* h) {
+  if (!h) return;
+  (void)hipSetDevice(h->cfg.device);
+  (void)hipStreamSynchronize(h->stream);
+  for (void* p : {(void*)h->d_logits, (void*)h->d_uniforms, (void*)h->d_ids, (void*)h->d_scores, (void*)h->d_topk_idx,
+                  (void*)h->d_topk_prob, (void*)h->d_workspace})
+    if (p) (void)hipFree(p);
+  if (h->ev0) (void)hipEventDestroy(h->ev0);
+  if (h->ev1) (void)hipEventDestroy(h->ev1);
+  if (h->owns_stream && h->stream) (void)hipStreamDestroy(h->stream);
+  delete h;
+}
+
+int mi355_sampler_sample(mi355_sampler* h, const float* logits, int32_t* ids, float* scores, char** error_msg) {
+  if (!ids) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null ids");
+  return run(h, logits, nullptr, ids, scores, nullptr, nullptr, true, error_msg);
+}
+
+int mi355_sampler_sample_with_uniforms(mi355_sampler* h, const float* logits, const float* uniforms, int32_t* ids,
+                                       float* scores, char** error_msg) {
+  if (!ids || !uniforms) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null ids or uniforms");
+  return run(h, logits, uniforms, ids, scores, nullptr, nullptr, false, error_msg);
+}
+
+int mi355_sampler_top_k(mi355_sampler* h, const float* logits, int32_t* indices, float* probabilities,
+                        char** error_msg) {
+  if (!indices || !probabilities)
+    return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null indices or probabilities");
+  return run(h, logits, nullptr, nullptr, nullptr, indices, probabilities, false, error_msg);
+}
+
+int mi355_sampler_sync(mi355_sampler* h, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_SAMPLER_INVALID_ARGUMENT, "null sampler");
+  HIP_OR_RETURN(hipSetDevice(h->cfg.device));
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+  return MI355_SAMPLER_OK;
+}
+
+int mi355_sampler_set_timing(mi355_sampler* h, int32_t enabled) {
+  if (!h) return MI355_SAMPLER_INVALID_ARGUMENT;
+  h->timing = enabled != 0;
+  if (!h->timing) h->timed = false;
+  return MI355_SAMPLER_OK;
+}
+
+float mi355_sampler_last_kernel_ms(mi355_sampler* h) {
+  if (!h || !h->timed) return -1.f;
+  if (hipEventSynchronize(h->ev1) != hipSuccess) return -1.f;
+  float ms = -1.f;
+  if (hipEventElapsedTime(&ms, h->ev0, h->ev1) != hipSuccess) return -1.f;
+  return ms;
+}
+
+}  // extern "C"
