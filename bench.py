@@ -67,15 +67,20 @@ def time_steps(torch, step_fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def kernel_ms(torch, at, step_fn, launches, first):
-    """Average duration of the attention kernel itself over `launches` calls."""
+def kernel_ms(torch, at, step_fn, launches, first, burst=8):
+    """Average duration of the attention kernel itself (begin / end stamps attached to
+    the dispatch) under the conditions of the timed region: steps are queued back to
+    back in bursts and the stamps of each burst's last launch are read."""
     at.set_timing(True)
-    total = 0.0
-    for i in range(launches):
-        step_fn(first + i)
+    total, n, i = 0.0, 0, first
+    while n < max(3, launches // burst):
+        for _ in range(burst):
+            step_fn(i)
+            i += 1
         total += at.last_kernel_ms()
+        n += 1
     at.set_timing(False)
-    return total / launches
+    return total / n
 
 
 def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, ctx=4096):
@@ -92,7 +97,7 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
         at.decode(r * layers, lens, q[r], out[r], num_splits=splits, n_layers=layers, batch=1)
 
     sec = time_steps(torch, step, steps, warmup)
-    kms = kernel_ms(torch, at, step, min(steps, 50), warmup + steps)
+    kms = kernel_ms(torch, at, step, steps, warmup + steps)
     # algorithmic bytes: K and V once, Q and O once (no partials, no padding)
     per_layer = ctx * hkv * D * 2 * 2 + 2 * hq * D * 2
     step_bytes = per_layer * layers
@@ -131,7 +136,7 @@ def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits
         at.decode(i % rotation, clens, q, out, num_splits=splits, batch=B)
 
     sec = time_steps(torch, step, steps, warmup)
-    kms = kernel_ms(torch, at, step, min(steps, 30), warmup + steps)
+    kms = kernel_ms(torch, at, step, steps, warmup + steps)
     esz = 1 if kv == A.I8 else 2
     nbytes = sum(lens) * hkv * D * 2 * esz + 2 * B * hq * D * 2 + (B * 2 * hkv * D * 4 if kv == A.I8 else 0)
     at.close()
@@ -159,7 +164,7 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False):
         at.prefill(0, 0, 0, n, q, out, n_layers=layers)
 
     sec = time_steps(torch, step, steps, warmup)
-    kms = kernel_ms(torch, at, step, min(steps, 30), 0)
+    kms = kernel_ms(torch, at, step, steps, 0)
     flops = sum(prefill_flops(n, hq, w) for w in windows)
 
     def step1(i):
@@ -190,7 +195,7 @@ def bench_decode_c1(A, torch, steps, warmup):
         at.decode(0, lens, q, out, num_splits=0, batch=1)
 
     sec = time_steps(torch, step, steps, warmup)
-    kms = kernel_ms(torch, at, step, min(steps, 30), 0)
+    kms = kernel_ms(torch, at, step, steps, 0)
     at.close()
     nbytes = ctx * hkv * D * 2 * 4 + 2 * hq * D * 4
     return {"workload": "C1: 1 seq x 1024, Hq4/Hkv1, fp32, one layer, cache-resident (latency)",
