@@ -10,18 +10,18 @@
 //
 // Two launches per call. select_kernel: a row of ~262k logits is cut into up to
 // 16 segments, one workgroup of 1024 threads each, so that one row already
-// spreads over 16 CUs. A workgroup finds the k largest of its segment in two
-// passes over it (the second one an L2 hit): every thread keeps the maximum of
-// the logits it reads; the k-th largest of those 1024 maxima is a lower bound of
-// the segment's k-th largest logit, so the second pass only has to collect what
-// reaches it - a few hundred candidates, which a bitonic sort in LDS orders
-// (descending value, equal values by ascending index). Segments for which that
-// bound is too weak (more than 2048 candidates: long runs of equal values) fall
-// back to a radix descent on an order-preserving 32-bit key with LDS histograms
-// (12 + 12 + 8 bits); exact ties at the k-th value are then taken in ascending
-// index order. finish_kernel: one workgroup per row merges the segments'
-// candidates by another sort and one thread walks the k winners in the
-// reference's op order.
+// spreads over 16 CUs. A workgroup reads its segment once, 16 logits per thread
+// that stay in registers. Every thread takes the maximum of its logits; every
+// wave reports the ceil(k/16)-th largest of its 64 maxima (DPP reductions); at
+// least k logits of the segment reach the smallest of those 16 numbers, so only
+// what reaches it - a few hundred candidates - is packed as (order-preserving
+// key, index) words, ranked by counting in LDS (no sort), and the segment's k
+// best go to a workspace. Segments for which that bound is too weak (more than
+// 2048 candidates: long runs of equal values) or that hold fewer than k numbers
+// fall back to a radix descent on the keys with LDS histograms (12 + 12 + 8
+// bits); exact ties at the k-th value are then taken in ascending index order.
+// finish_kernel: one workgroup per row merges the segments' candidates the same
+// way and walks the k winners in the reference's op order.
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <float.h>
@@ -165,6 +165,21 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
+// The same for floats; -inf is the identity, NaN never wins (v_max_f32 returns the other operand).
+__device__ __forceinline__ float wave_max_f32(float v) {
+  const int ninf = 0xff800000;
+#define MI355_DPP_FMAX(ctrl, row_mask) \
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), ctrl, row_mask, 0xf, false)))
+  MI355_DPP_FMAX(0x111, 0xf);
+  MI355_DPP_FMAX(0x112, 0xf);
+  MI355_DPP_FMAX(0x114, 0xf);
+  MI355_DPP_FMAX(0x118, 0xf);
+  MI355_DPP_FMAX(0x142, 0xa);
+  MI355_DPP_FMAX(0x143, 0xc);
+#undef MI355_DPP_FMAX
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 // A lower bound that at least k of the values v (one per thread, 0 = none) reach:
 // every wave reports the j-th largest of its 64 values, j = ceil(k / 16); at
 // least 16 j >= k values reach the smallest of those 16 numbers. One barrier.
@@ -184,14 +199,35 @@ __device__ __forceinline__ uint32_t lower_bound_of_kth(uint32_t v, int k, uint32
   return tau;
 }
 
+// The float version (-inf = none): used on the logits themselves.
+__device__ __forceinline__ float lower_bound_of_kth_f32(float v, int k, float* wave_val, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  const int j_th = (k + kWavesPerWg - 1) / kWavesPerWg;
+  float m = -INFINITY;
+  for (int r = 0; r < j_th; ++r) {
+    m = wave_max_f32(v);
+    const u64 holders = __ballot(v == m);
+    if (lane == __ffsll((long long)holders) - 1) v = -INFINITY;  // drop one holder of the maximum
+  }
+  if (lane == 0) wave_val[wave] = m;
+  __syncthreads();
+  float tau = wave_val[0];
+  for (int w = 1; w < kWavesPerWg; ++w) tau = fminf(tau, wave_val[w]);
+  return tau;
+}
+
 // top[r] = the candidate of rank r (number of larger candidates; the words are
 // distinct) for r < k, by counting instead of sorting: 256 candidates at a
 // time, the comparisons of each split over 4 threads.
 __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, int k, uint32_t* rank_sm, int tid) {
-  const int slot = tid & 255, part = tid >> 8;
-  const int span = (n + 3) / 4, j0 = part * span, j1 = min(n, j0 + span);
-  for (int blk = 0; blk < n; blk += 256) {
-    if (tid < 256) rank_sm[tid] = 0;
+  // `width` candidates at a time (a power of two, 128 .. 1024), the comparisons of each split over 1024 / width threads
+  int width = 128;
+  while (width < n && width < kThreads) width <<= 1;
+  const int parts = kThreads / width;
+  const int slot = tid & (width - 1), part = tid / width;
+  const int span = (n + parts - 1) / parts, j0 = part * span, j1 = min(n, j0 + span);
+  for (int blk = 0; blk < n; blk += width) {
+    if (tid < width) rank_sm[tid] = 0;
     __syncthreads();
     if (blk + slot < n) {
       const u64 c = cand[blk + slot];
@@ -206,7 +242,7 @@ __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, in
       if (cnt) atomicAdd(&rank_sm[slot], cnt);
     }
     __syncthreads();
-    if (tid < 256 && blk + tid < n && rank_sm[tid] < (uint32_t)k) top[rank_sm[tid]] = cand[blk + tid];
+    if (tid < width && blk + tid < n && rank_sm[tid] < (uint32_t)k) top[rank_sm[tid]] = cand[blk + tid];
     __syncthreads();
   }
 }
@@ -216,7 +252,7 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
   __shared__ uint32_t hist[kBins];
   __shared__ u64 cand[kCap];
   __shared__ u64 top[kMaxK];
-  __shared__ uint32_t rank_sm[256];
+  __shared__ uint32_t rank_sm[kThreads];
   __shared__ uint32_t wave_sum[kWavesPerWg];
   __shared__ uint32_t found[3];  // bin, count above it, count in it
   __shared__ uint32_t n_cand, n_ties;
@@ -230,20 +266,21 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
   const bool vec_ok = (a.vocab % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
   u64* out = a.workspace + ((size_t)b * a.segments + sgm) * a.k;
 
-  // A segment of up to 16 logits per thread is read from memory once: its keys
-  // stay in registers for all later passes (same index layout as for_each_key).
+  // A segment of up to 16 logits per thread is read from memory once and stays in
+  // registers for all later passes (same index layout as for_each_key); slots past
+  // the segment's end hold NaN, which no comparison and no maximum ever picks.
   const bool resident = len <= kThreads * kResident;
-  uint32_t kreg[kResident];
+  float xreg[kResident];
   if (resident) {
 #pragma unroll
     for (int u = 0; u < kResident / 4; ++u) {
       const int base = u * kPerIter + tid * 4;
       if (vec_ok && base + 3 < len) {
         const float4 x = *reinterpret_cast<const float4*>(seg + base);
-        kreg[4 * u] = key_of(x.x); kreg[4 * u + 1] = key_of(x.y); kreg[4 * u + 2] = key_of(x.z); kreg[4 * u + 3] = key_of(x.w);
+        xreg[4 * u] = x.x; xreg[4 * u + 1] = x.y; xreg[4 * u + 2] = x.z; xreg[4 * u + 3] = x.w;
       } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) kreg[4 * u + j] = base + j < len ? key_of(seg[base + j]) : 0u;
+        for (int j = 0; j < 4; ++j) xreg[4 * u + j] = base + j < len ? seg[base + j] : __int_as_float(0x7fc00000);
       }
     }
   }
@@ -254,7 +291,7 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int i = u * kPerIter + tid * 4 + j;
-          if (i < len) f(kreg[4 * u + j], i);
+          if (i < len) f(key_of(xreg[4 * u + j]), i);
         }
     } else {
       for_each_key(seg, len, vec_ok, tid, f);
@@ -278,7 +315,29 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
   }
 
   // ---- a threshold from the per-thread maxima, then everything that reaches it
-  {
+  if (resident) {
+    // on the logits themselves: three instructions per logit, keys only for the candidates
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < kResident; ++e) tmax = fmaxf(tmax, xreg[e]);
+    if (tid == 0) n_cand = 0;
+    const float tau = lower_bound_of_kth_f32(tmax, k, reinterpret_cast<float*>(wave_sum), tid);  // (barrier inside)
+    uint32_t mine = 0;
+#pragma unroll
+    for (int e = 0; e < kResident; ++e) mine += xreg[e] >= tau ? 1u : 0u;
+    uint32_t pos = mine ? atomicAdd(&n_cand, mine) : 0u;
+    if (mine) {
+#pragma unroll
+      for (int u = 0; u < kResident / 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (xreg[4 * u + j] >= tau) {
+            if (pos < (uint32_t)kCap) cand[pos] = pack(key_of(xreg[4 * u + j]), index0 + u * kPerIter + tid * 4 + j);
+            ++pos;
+          }
+    }
+    __syncthreads();
+  } else {
     uint32_t tmax = 0;
     each([&](uint32_t key, int) { tmax = max(tmax, key); });
     if (tid == 0) n_cand = 0;
@@ -294,7 +353,7 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
     });
     __syncthreads();
   }
-  const bool fast_ok = n_cand <= (uint32_t)kCap;
+  const bool fast_ok = n_cand <= (uint32_t)kCap && n_cand >= (uint32_t)k;  // (fewer than k: NaNs among the logits)
   __syncthreads();
 
   if (!fast_ok) {
@@ -374,7 +433,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
   __shared__ u64 surv[kMergeCap];  // the segments' candidates that reach the threshold
   __shared__ u64 cand[kMaxK];      // the row's k winners, descending
   __shared__ float e_sm[kMaxK];
-  __shared__ uint32_t rank_sm[256];
+  __shared__ uint32_t rank_sm[kThreads];
   __shared__ uint32_t wave_val[kWavesPerWg];
   __shared__ uint32_t n_surv;
   __shared__ float inv_sm;
