@@ -248,7 +248,12 @@ __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, in
 }
 
 // The k largest logits of one segment of one row, sorted, into the workspace.
-__global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
+// RESIDENT: every segment has at most kSegmentMin logits (the host knows), which
+// then stay in registers; the other instantiation re-reads them (from L2) per pass.
+// 64 registers at most, so that two workgroups share a compute unit.
+template <bool RESIDENT>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
+select_kernel(const SamplerArgs a) {
   __shared__ uint32_t hist[kBins];
   __shared__ u64 cand[kCap];
   __shared__ u64 top[kMaxK];
@@ -269,9 +274,9 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
   // A segment of up to 16 logits per thread is read from memory once and stays in
   // registers for all later passes (same index layout as for_each_key); slots past
   // the segment's end hold NaN, which no comparison and no maximum ever picks.
-  const bool resident = len <= kThreads * kResident;
-  float xreg[kResident];
-  if (resident) {
+  constexpr bool resident = RESIDENT;
+  float xreg[RESIDENT ? kResident : 1];
+  if constexpr (resident) {
 #pragma unroll
     for (int u = 0; u < kResident / 4; ++u) {
       const int base = u * kPerIter + tid * 4;
@@ -285,7 +290,7 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
     }
   }
   auto each = [&](auto&& f) {
-    if (resident) {
+    if constexpr (resident) {
 #pragma unroll
       for (int u = 0; u < kResident / 4; ++u)
 #pragma unroll
@@ -315,7 +320,7 @@ __global__ void __launch_bounds__(kThreads) select_kernel(const SamplerArgs a) {
   }
 
   // ---- a threshold from the per-thread maxima, then everything that reaches it
-  if (resident) {
+  if constexpr (resident) {
     // on the logits themselves: three instructions per logit, keys only for the candidates
     float tmax = -INFINITY;
 #pragma unroll
@@ -612,8 +617,12 @@ int run(mi355_sampler* h, const float* logits, const float* uniforms, int32_t* i
   a.segments = h->segments;
   a.seg_len = h->seg_len;
   // ev0 / ev1 ride on the dispatches: begin of the first kernel, end of the second
-  hipExtLaunchKernelGGL(select_kernel, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
-                        h->timing ? h->ev0 : nullptr, nullptr, 0, a);
+  if (h->seg_len <= kSegmentMin)
+    hipExtLaunchKernelGGL(select_kernel<true>, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
+                          h->timing ? h->ev0 : nullptr, nullptr, 0, a);
+  else
+    hipExtLaunchKernelGGL(select_kernel<false>, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
+                          h->timing ? h->ev0 : nullptr, nullptr, 0, a);
   HIP_OR_RETURN(hipGetLastError());
   hipExtLaunchKernelGGL(finish_kernel, dim3((unsigned)B), dim3(kThreads), 0, h->stream, nullptr,
                         h->timing ? h->ev1 : nullptr, 0, a);

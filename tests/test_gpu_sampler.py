@@ -87,7 +87,7 @@ def test_reference_held_values():
     say("sampler: reference-held values ok")
 
 
-@pytest.mark.parametrize("vocab,k", [(262144, 64), (262144, 40), (32000, 256), (50257, 8), (1000, 1000), (7, 3), (4099, 2)])
+@pytest.mark.parametrize("vocab,k", [(262144, 64), (300001, 50), (524288, 256), (262144, 40), (32000, 256), (50257, 8), (1000, 1000), (7, 3), (4099, 2)])
 def test_top_k_and_probabilities_match_oracle(vocab, k):
     rng = np.random.default_rng(vocab + k)
     b = 5
@@ -110,7 +110,7 @@ def test_top_k_and_probabilities_match_oracle(vocab, k):
 def test_all_equal_and_fallback_paths():
     # every logit equal: the bound from the thread maxima admits the whole row -> radix descent,
     # exact ties taken in ascending index order
-    for vocab in (262144, 5000, 70000):
+    for vocab in (262144, 5000, 70000, 400000):
         for value in (0.0, -3.5, 7.25):
             logits = np.full((2, vocab), value, np.float32)
             logits[1, vocab - 5:] = value + 1.0     # five winners at the very end, then ties from index 0
