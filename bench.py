@@ -248,6 +248,45 @@ def bench_sampler(S, torch, steps, warmup, batch=64, vocab=262144, k=64, p=0.95,
             "tokens_per_s": batch / sec, "single_row_latency_us": lat * 1e6}
 
 
+def bench_pre_attention(A, torch, steps, warmup, layers=26, n=1024, hq=4, hkv=1):
+    """The step before attention at config 2's shape: per layer one launch that RMS-normalises
+    and rotates the chunk's q / k rows and writes k / v into the cache planes (bf16). Every
+    step takes the next layer (its own inputs and planes), as a forward pass does."""
+    dt = torch.bfloat16
+    g = torch.Generator(device="cuda:0").manual_seed(0xC0FFEE + 8)
+    mk = lambda heads: [torch.randn((n, heads, D), generator=g, device="cuda:0").to(dt) for _ in range(layers)]
+    q, k, v = mk(hq), mk(hkv), mk(hkv)
+    q_out = torch.zeros_like(q[0])
+    rng = np.random.default_rng(0xC0FFEE + 8)
+    d = np.arange(0, D, 2, dtype=np.float64) / D
+    with A.Attn(layers, hq, hkv, D, n, 1, A.BF16, A.BF16, stream=torch.cuda.current_stream().cuda_stream) as at:
+        for layer in range(layers):
+            theta = 1000000.0 if (layer + 1) % 6 == 0 else 10000.0
+            at.set_layer_transform(layer, norm_q=True, norm_k=True,
+                                   q_weight=(rng.standard_normal(D) * 0.1).astype(np.float32),
+                                   k_weight=(rng.standard_normal(D) * 0.1).astype(np.float32), eps=1e-6,
+                                   weight_offset=1.0, rope_inv_freq=(theta ** -d).astype(np.float32))
+
+        def step(i):
+            layer = i % layers
+            at.pre_attention(layer, 0, 0, q[layer], k[layer], v[layer], q_out)
+        sec = time_steps(torch, step, steps, warmup)
+        kms = kernel_ms(torch, at, step, steps, warmup + steps)
+    with A.Attn(1, 8, 2, D, 4096, 1, A.F16, A.F16, stream=torch.cuda.current_stream().cuda_stream) as at1:
+        at1.set_layer_transform(0, norm_q=True, norm_k=True, eps=1e-6, rope_inv_freq=(10000.0 ** -d).astype(np.float32))
+        q1 = torch.randn((1, 8, D), generator=g, device="cuda:0").half()
+        k1 = torch.randn((1, 2, D), generator=g, device="cuda:0").half()
+        o1 = torch.zeros_like(q1)
+        lat = time_steps(torch, lambda i: at1.pre_attention(0, 0, 100 + i % 3000, q1, k1, k1, o1), 200, 20)
+    nbytes = 2 * n * (hq + 2 * hkv) * D * 2  # every row read once and written once
+    return {"workload": f"step before attention, config 2 shape: {n} tokens x (Hq{hq} + 2 x Hkv{hkv}) rows, bf16, "
+                        f"RMS norm of q / k + rotary embedding + cache write, one launch per layer, {layers} layers in turn "
+                        "(6 MiB per launch: L2 / Infinity Cache resident, launch-latency bound)",
+            "ms_per_step": sec * 1e3, "kernel_ms": kms, "bytes": nbytes, "GBps": nbytes / sec / 1e9,
+            "kernel_GBps": nbytes / (kms * 1e-3) / 1e9, "tokens_per_s": n / sec,
+            "single_token_latency_us": lat * 1e6}
+
+
 def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=12.0):
     """C restatement of the reference CPU op order (fp32, OpenMP) on the same
     30-layer decode sweep, repeated until about `budget_s` seconds are spent."""
@@ -379,6 +418,10 @@ def main():
         log(f"[bench] {smp['workload']}: {smp['ms_per_step']*1e3:.1f} us/step, kernel {smp['kernel_GBps']:.0f} GB/s, "
             f"one row {smp['single_row_latency_us']:.1f} us")
         result["sampler"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in smp.items()}
+        pa = bench_pre_attention(A, torch, args.steps, args.warmup)
+        log(f"[bench] {pa['workload']}: {pa['ms_per_step']*1e3:.1f} us/step, kernel {pa['kernel_ms']*1e3:.1f} us "
+            f"({pa['kernel_GBps']:.0f} GB/s), one token {pa['single_token_latency_us']:.1f} us")
+        result["pre_attention"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in pa.items()}
 
     if not args.no_cpu:
         cpu = cpu_baseline_c3(dec["layers"], 4096, dec["step_bytes"])

@@ -111,6 +111,58 @@ int mi355_attn_kv_append(mi355_attn* handle, int32_t layer, int32_t seq, int32_t
 int mi355_attn_kv_set_scales(mi355_attn* handle, int32_t layer, int32_t seq, const float* k_scale,
                              const float* v_scale, char** error_msg);
 
+/*
+ * Per-layer constants of the step before attention (mi355_attn_pre_attention).
+ * All pointers are HOST arrays (whatever host_io says), copied before the call
+ * returns. In the reference these are weights and tables of the model graph:
+ * the NPU flow computes the rotary cos / sin tables for local and global layers
+ * from `input_pos` in a signature of its own
+ * (llm_litert_npu_compiled_model_executor.cc:82-94,1209-1219), the norms sit in
+ * the transformer stack behind compiled_model_.Run.
+ *   RMS norm over head_dim:  y = x / sqrt(mean(x^2) + eps) * (weight_offset + weight[d])
+ *                            (weight NULL: no learned scale; Gemma 3: weight_offset 1)
+ *   rotary embedding:        angle = float32(position) * rope_inv_freq[d], d < head_dim/2;
+ *                            (x[d], x[d + head_dim/2]) is rotated by angle
+ *                            (the "rotate half" pairing; rope_inv_freq NULL: no rotation).
+ *                            A global layer passes theta^(-2d/head_dim) / factor of its
+ *                            own theta, a local layer that of the local theta.
+ */
+typedef struct mi355_attn_layer_transform {
+  uint32_t struct_size;       /* sizeof(mi355_attn_layer_transform) */
+  int32_t norm_q;             /* != 0: RMS-normalise every query head */
+  int32_t norm_k;             /* != 0: RMS-normalise every key head */
+  int32_t norm_v;             /* != 0: RMS-normalise every value head, no learned scale */
+  const float* q_weight;      /* [head_dim] or NULL */
+  const float* k_weight;      /* [head_dim] or NULL */
+  float eps;                  /* >= 0 */
+  float weight_offset;
+  const float* rope_inv_freq; /* [head_dim / 2] or NULL */
+} mi355_attn_layer_transform;
+
+/* Sets the constants of one layer; waits for the work queued on the handle first. */
+int mi355_attn_set_layer_transform(mi355_attn* handle, int32_t layer, const mi355_attn_layer_transform* transform,
+                                   char** error_msg);
+
+/*
+ * The step before attention for n new tokens of one layer of sequence `seq` at
+ * positions pos .. pos+n-1, in one launch: RMS norm of q / k (/ v), rotary
+ * embedding of q and k (as set by mi355_attn_set_layer_transform; a layer
+ * without constants gets neither), q_out = the query rows attention reads
+ * (io_dtype, may be q itself), and the key / value rows written into the cache
+ * exactly as mi355_attn_kv_append would write them.
+ * q [n][num_q_heads][head_dim], k, v [n][num_kv_heads][head_dim], all io_dtype.
+ * int8 cache: the rows are quantised with the scales set by
+ * mi355_attn_kv_set_scales, value = clamp(round(x * (1 / scale)), -127, 127)
+ * (round half away from zero; a zero scale stores 0).
+ * Replaces: the RoPE and cache-update signatures of the NPU flow
+ * (llm_litert_npu_compiled_model_executor.cc:82-110,1209-1219,1294-1333) and
+ * its float -> integer quantise step (:116-148); in the CPU/GPU executor the
+ * same work is inside compiled_model_.Run
+ * (llm_litert_compiled_model_executor.cc:271,407,522).
+ */
+int mi355_attn_pre_attention(mi355_attn* handle, int32_t layer, int32_t seq, int32_t pos, int32_t n,
+                             const void* q, const void* k, const void* v, void* q_out, char** error_msg);
+
 /* Reads cache rows pos .. pos+n-1 back in boundary layout (tests, debugging). */
 int mi355_attn_kv_read(mi355_attn* handle, int32_t layer, int32_t seq, int32_t pos, int32_t n, void* k_out,
                        void* v_out, char** error_msg);
@@ -170,8 +222,8 @@ int mi355_attn_sync(mi355_attn* handle, char** error_msg);
 void* mi355_attn_stream(mi355_attn* handle);
 
 /*
- * Duration in milliseconds of the attention kernel of the most recent
- * prefill/decode call, measured with HIP events on the handle's stream
+ * Duration in milliseconds of the kernel of the most recent
+ * prefill / decode / pre_attention call, measured with HIP events on the handle's stream
  * (the split-merge pass is excluded). Blocks until that call has finished.
  * Timing is recorded only after mi355_attn_set_timing(handle, 1).
  */

@@ -48,6 +48,21 @@ class Config(ctypes.Structure):
     ]
 
 
+class LayerTransform(ctypes.Structure):
+    """mi355_attn_layer_transform: the constants of the step before attention."""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("norm_q", ctypes.c_int32),
+        ("norm_k", ctypes.c_int32),
+        ("norm_v", ctypes.c_int32),
+        ("q_weight", ctypes.c_void_p),
+        ("k_weight", ctypes.c_void_p),
+        ("eps", ctypes.c_float),
+        ("weight_offset", ctypes.c_float),
+        ("rope_inv_freq", ctypes.c_void_p),
+    ]
+
+
 _ERR = ctypes.POINTER(ctypes.c_char_p)
 
 
@@ -70,6 +85,8 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_kv_append.argtypes = [vp, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_kv_set_scales.argtypes = [vp, i32, i32, vp, vp, errp]
     L.mi355_attn_kv_read.argtypes = [vp, i32, i32, i32, i32, vp, vp, errp]
+    L.mi355_attn_set_layer_transform.argtypes = [vp, i32, ctypes.POINTER(LayerTransform), errp]
+    L.mi355_attn_pre_attention.argtypes = [vp, i32, i32, i32, i32, vp, vp, vp, vp, errp]
     L.mi355_attn_prefill.argtypes = [vp, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_prefill_layers.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_decode.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
@@ -177,6 +194,32 @@ class Attn:
         err = ctypes.c_void_p()
         _check(lib().mi355_attn_kv_read(self._h, layer, seq, pos, n, _ptr(k_out), _ptr(v_out), ctypes.byref(err)),
                err)
+
+    def set_layer_transform(self, layer, *, norm_q=False, norm_k=False, norm_v=False, q_weight=None, k_weight=None,
+                            eps=1e-6, weight_offset=1.0, rope_inv_freq=None):
+        """Constants of the step before attention for one layer; the arrays are
+        host float32 ([head_dim] weights, [head_dim / 2] rotary frequencies)."""
+        def host(x, count, name):
+            if x is None:
+                return None
+            arr = np.ascontiguousarray(np.asarray(x, dtype=np.float32))
+            if arr.shape != (count,):
+                raise ValueError(f"{name} must hold {count} float32 values")
+            return arr
+        qw, kw = host(q_weight, self.d, "q_weight"), host(k_weight, self.d, "k_weight")
+        fr = host(rope_inv_freq, self.d // 2, "rope_inv_freq")
+        t = LayerTransform(ctypes.sizeof(LayerTransform), int(bool(norm_q)), int(bool(norm_k)), int(bool(norm_v)),
+                           _ptr(qw), _ptr(kw), float(eps), float(weight_offset), _ptr(fr))
+        err = ctypes.c_void_p()
+        _check(lib().mi355_attn_set_layer_transform(self._h, layer, ctypes.byref(t), ctypes.byref(err)), err)
+
+    def pre_attention(self, layer, seq, pos, q, k, v, q_out, n=None):
+        """Norm + rotary embedding of the n new rows, query into q_out, key /
+        value rows into the cache (the step before prefill / decode)."""
+        n = int(q.shape[0]) if n is None else n
+        err = ctypes.c_void_p()
+        _check(lib().mi355_attn_pre_attention(self._h, layer, seq, pos, n, _ptr(q), _ptr(k), _ptr(v), _ptr(q_out),
+                                              ctypes.byref(err)), err)
 
     # -- attention
     def prefill(self, layer, seq, q_pos0, n, q, out, n_layers=1):

@@ -142,5 +142,24 @@ struct KvCopyArgs {
   void* v;
 };
 
+// Per-layer constants of the step before attention, float32 in HBM:
+// [head_dim / 2] rotary frequencies, [head_dim] query norm weights, [head_dim] key norm weights.
+MI355_HD int transform_floats(int head_dim) { return head_dim / 2 + 2 * head_dim; }
+
+// Arguments of pre_attention_kernel (norm + rotary embedding + cache write).
+struct PreAttentionArgs {
+  const void* q;   // [n][hq][D] io dtype
+  const void* k;   // [n][hkv][D] io dtype
+  const void* v;   // [n][hkv][D] io dtype
+  void* q_out;     // [n][hq][D] io dtype (may be q)
+  uint8_t* cache;
+  const float* scales;     // int8 cache: [layer][seq][K/V][hkv][D]
+  const float* constants;  // this layer's transform_floats(D) floats
+  CacheGeom geom;
+  int32_t layer, seq, pos, n, hq;
+  int32_t rope, norm_q, norm_k, norm_v, q_scaled, k_scaled;  // flags
+  float eps, weight_offset;
+};
+
 }  // namespace mi355
 #endif  // LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_

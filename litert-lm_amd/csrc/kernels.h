@@ -29,5 +29,10 @@ hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, h
 hipError_t launch_kv_append(const KvCopyArgs& args, hipStream_t stream);
 hipError_t launch_kv_read(const KvCopyArgs& args, hipStream_t stream);
 
+// Norm + rotary embedding of n new rows, query written out, key / value rows
+// written into the cache planes (quantised for an int8 cache).
+hipError_t launch_pre_attention(const PreAttentionArgs& args, int kv_dtype, int io_dtype, hipStream_t stream,
+                                hipEvent_t ev0, hipEvent_t ev1);
+
 }  // namespace mi355
 #endif  // LITERT_LM_AMD_CSRC_KERNELS_H_

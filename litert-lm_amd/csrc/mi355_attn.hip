@@ -11,6 +11,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <cmath>
 #include <new>
 #include <string>
 #include <vector>
@@ -70,6 +71,13 @@ struct mi355_attn {
   float* scales = nullptr;
   int32_t* d_window = nullptr;
   int32_t* d_sched = nullptr;  // prefill work-queue counters
+  // the step before attention: per-layer constants in HBM and what is switched on
+  struct LayerTransform {
+    bool set = false, rope = false, norm_q = false, norm_k = false, norm_v = false, q_scaled = false, k_scaled = false;
+    float eps = 1e-6f, weight_offset = 1.f;
+  };
+  float* d_transform = nullptr;  // [num_layers][transform_floats(head_dim)]
+  std::vector<LayerTransform> transform;
   std::vector<int32_t> window;
   std::vector<int32_t> filled;  // [layer][seq] rows written since the last reset
   // split-KV workspace
@@ -449,6 +457,12 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
     return bail(MI355_ATTN_INTERNAL, "window upload", e);
   if ((e = hipMalloc(&h->d_sched, sizeof(int32_t) * kPrefillSchedInts)) != hipSuccess)
     return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "prefill queue counters", e);
+  h->transform.assign(c->num_layers, mi355_attn::LayerTransform{});
+  const size_t transform_bytes = sizeof(float) * (size_t)c->num_layers * transform_floats(c->head_dim);
+  if ((e = hipMalloc(&h->d_transform, transform_bytes)) != hipSuccess)
+    return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "layer transform constants", e);
+  if ((e = hipMemsetAsync(h->d_transform, 0, transform_bytes, h->stream)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "layer transform clear", e);
   if ((e = hipMemsetAsync(h->d_sched, 0, sizeof(int32_t) * kPrefillSchedInts, h->stream)) != hipSuccess)
     return bail(MI355_ATTN_INTERNAL, "prefill queue clear", e);
   h->ring_slot_ints = 2 * c->max_seqs;
@@ -474,6 +488,7 @@ void mi355_attn_destroy(mi355_attn* h) {
   if (h->scales) (void)hipFree(h->scales);
   if (h->d_window) (void)hipFree(h->d_window);
   if (h->d_sched) (void)hipFree(h->d_sched);
+  if (h->d_transform) (void)hipFree(h->d_transform);
   if (h->ws_acc) (void)hipFree(h->ws_acc);
   if (h->ws_ml) (void)hipFree(h->ws_ml);
   if (h->d_ring) (void)hipFree(h->d_ring);
@@ -539,6 +554,93 @@ int mi355_attn_kv_set_scales(mi355_attn* h, int32_t layer, int32_t seq, const fl
                                h->stream));
   if (h->cfg.host_io) HIP_OR_RETURN(hipStreamSynchronize(h->stream));
   return MI355_ATTN_OK;
+}
+
+int mi355_attn_set_layer_transform(mi355_attn* h, int32_t layer, const mi355_attn_layer_transform* t,
+                                   char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (!t || t->struct_size != sizeof(mi355_attn_layer_transform))
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null transform or struct_size mismatch");
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (!(t->eps >= 0.f) || !std::isfinite(t->eps) || !std::isfinite(t->weight_offset))
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "eps %g must be finite and >= 0, weight_offset %g finite",
+                (double)t->eps, (double)t->weight_offset);
+  const int D = h->cfg.head_dim;
+  if (t->rope_inv_freq)
+    for (int d = 0; d < D / 2; ++d)
+      if (!std::isfinite(t->rope_inv_freq[d]))
+        return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "rope_inv_freq[%d] is not finite", d);
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  // the constants are host arrays whatever host_io says; copied before this call returns
+  std::vector<float> row((size_t)transform_floats(D), 0.f);
+  if (t->rope_inv_freq) memcpy(row.data(), t->rope_inv_freq, sizeof(float) * (D / 2));
+  if (t->q_weight) memcpy(row.data() + D / 2, t->q_weight, sizeof(float) * D);
+  if (t->k_weight) memcpy(row.data() + D / 2 + D, t->k_weight, sizeof(float) * D);
+  HIP_OR_RETURN(hipStreamSynchronize(h->stream));  // earlier launches may still read the old constants
+  HIP_OR_RETURN(hipMemcpy(h->d_transform + (size_t)layer * transform_floats(D), row.data(), sizeof(float) * row.size(),
+                          hipMemcpyHostToDevice));
+  mi355_attn::LayerTransform& lt = h->transform[layer];
+  lt.set = true;
+  lt.rope = t->rope_inv_freq != nullptr;
+  lt.norm_q = t->norm_q != 0;
+  lt.norm_k = t->norm_k != 0;
+  lt.norm_v = t->norm_v != 0;
+  lt.q_scaled = lt.norm_q && t->q_weight != nullptr;
+  lt.k_scaled = lt.norm_k && t->k_weight != nullptr;
+  lt.eps = t->eps;
+  lt.weight_offset = t->weight_offset;
+  return MI355_ATTN_OK;
+}
+
+int mi355_attn_pre_attention(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos, int32_t n, const void* q,
+                             const void* k, const void* v, void* q_out, char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (seq < 0 || seq >= h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq %d outside [0, %d)", seq, h->cfg.max_seqs);
+  if (n < 0 || pos < 0 || (int64_t)pos + n > h->cfg.max_tokens)
+    return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "rows [%d, %lld) outside [0, max_tokens=%d]", pos,
+                (long long)pos + n, h->cfg.max_tokens);
+  if (n == 0) return MI355_ATTN_OK;
+  if (!q || !k || !v || !q_out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null q, k, v or q_out");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  const size_t q_bytes = (size_t)n * h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
+  const size_t kv_bytes = (size_t)n * h->cfg.num_kv_heads * h->cfg.head_dim * io_size(h);
+  const void *dq = nullptr, *dk = nullptr, *dv = nullptr;
+  void* dout = nullptr;
+  if (int rc = stage_in(h, 0, q, q_bytes, &dq, error_msg)) return rc;
+  if (int rc = stage_in(h, 2, k, kv_bytes, &dk, error_msg)) return rc;
+  if (int rc = stage_in(h, 3, v, kv_bytes, &dv, error_msg)) return rc;
+  if (int rc = stage_out_begin(h, 1, q_out, q_bytes, &dout, error_msg)) return rc;
+  const mi355_attn::LayerTransform& lt = h->transform[layer];  // never set: a plain append
+  PreAttentionArgs a{};
+  a.q = dq;
+  a.k = dk;
+  a.v = dv;
+  a.q_out = dout;
+  a.cache = h->cache;
+  a.scales = h->scales;
+  a.constants = h->d_transform + (size_t)layer * transform_floats(h->cfg.head_dim);
+  a.geom = h->geom;
+  a.layer = layer;
+  a.seq = seq;
+  a.pos = pos;
+  a.n = n;
+  a.hq = h->cfg.num_q_heads;
+  a.rope = lt.rope;
+  a.norm_q = lt.norm_q;
+  a.norm_k = lt.norm_k;
+  a.norm_v = lt.norm_v;
+  a.q_scaled = lt.q_scaled;
+  a.k_scaled = lt.k_scaled;
+  a.eps = lt.eps;
+  a.weight_offset = lt.weight_offset;
+  HIP_OR_RETURN(launch_pre_attention(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, h->timing ? h->ev0 : nullptr,
+                                     h->timing ? h->ev1 : nullptr));
+  h->timed = h->timing;
+  int32_t& f = h->filled[(size_t)layer * h->cfg.max_seqs + seq];
+  f = std::max(f, pos + n);
+  return stage_out_end(h, 1, q_out, q_bytes, error_msg);
 }
 
 int mi355_attn_kv_read(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos, int32_t n, void* k_out, void* v_out,

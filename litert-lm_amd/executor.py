@@ -29,7 +29,7 @@ class _Config(ctypes.Structure):
         ("runner_lengths", ctypes.POINTER(ctypes.c_int32)),
         ("num_runners", ctypes.c_int32), ("fp16_activations", ctypes.c_int32),
         ("recording_backend", ctypes.c_int32), ("execute_pending_on_single_id_chunk", ctypes.c_int32),
-        ("softcap", ctypes.c_float),
+        ("softcap", ctypes.c_float), ("pre_attention", ctypes.c_int32),
     ]
 
 
@@ -80,13 +80,13 @@ class HipLlmExecutor:
 
     def __init__(self, num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens, runner_lengths=(1024,),
                  layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=True,
-                 softcap=0.0):
+                 softcap=0.0, pre_attention=False):
         self._win = _arr(layer_window) if layer_window is not None else None
         self._runners = _arr(runner_lengths)
         cfg = _Config(num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens,
                       ctypes.cast(self._win, ctypes.POINTER(ctypes.c_int32)) if self._win is not None else None,
                       ctypes.cast(self._runners, ctypes.POINTER(ctypes.c_int32)), len(runner_lengths), int(fp16),
-                      int(recording_backend), int(execute_pending_on_single_id_chunk), softcap)
+                      int(recording_backend), int(execute_pending_on_single_id_chunk), softcap, int(pre_attention))
         self._h = ctypes.c_void_p()
         err = ctypes.c_void_p()
         _check(lib().hle_create(ctypes.byref(cfg), ctypes.byref(self._h), ctypes.byref(err)), err)

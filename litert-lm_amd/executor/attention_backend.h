@@ -18,6 +18,18 @@ struct mi355_attn;
 
 namespace litert::lm {
 
+// Constants of the step right before attention for one layer: RMS norm of the
+// query / key (/ value) heads and the rotary embedding (in the reference part of
+// the model graph; the NPU flow runs the rotary tables and the cache update as
+// signatures of their own, llm_litert_npu_compiled_model_executor.cc:82-110).
+struct LayerTransform {
+  bool norm_q = false, norm_k = false, norm_v = false;
+  std::vector<float> q_weight, k_weight;  // [head_dim] or empty: no learned scale
+  float eps = 1e-6f;
+  float weight_offset = 1.f;              // learned scale = weight_offset + weight
+  std::vector<float> rope_inv_freq;       // [head_dim / 2] or empty: no rotation
+};
+
 struct AttentionShape {
   int num_layers = 0;
   int num_q_heads = 0;
@@ -27,6 +39,7 @@ struct AttentionShape {
   std::vector<int> layer_window;  // per layer, 0 = global
   float scale = 0.f;              // 0 => head_dim^-0.5
   float softcap = 0.f;
+  std::vector<LayerTransform> transforms;  // per layer; empty = the layers hand over finished q / k / v rows
 };
 
 class AttentionBackend {
@@ -34,6 +47,9 @@ class AttentionBackend {
   virtual ~AttentionBackend() = default;
   // k, v: [n][kv_heads][head_dim] float32 host rows written at pos .. pos+n-1.
   virtual Status Append(int layer, int pos, int n, const float* k, const float* v) = 0;
+  // The same with the layer's transform applied first: q [n][q_heads][head_dim] is
+  // normalised and rotated in place, k / v go through norm / rotation into the cache.
+  virtual Status PreAttention(int layer, int pos, int n, float* q, const float* k, const float* v) = 0;
   // q, out: [n][q_heads][head_dim] float32 host; rows at positions q_pos0 .. q_pos0+n-1.
   virtual Status Prefill(int layer, int q_pos0, int n, const float* q, float* out) = 0;
   // One row at position kv_len - 1.
@@ -54,6 +70,9 @@ class RecordingAttentionBackend : public AttentionBackend {
     if (pos + n > shape_.max_tokens) return OutOfRangeError("KV cache is full.");
     calls.push_back({AttentionCall::kAppend, layer, pos, n});
     return OkStatus();
+  }
+  Status PreAttention(int layer, int pos, int n, float*, const float* k, const float* v) override {
+    return Append(layer, pos, n, k, v);
   }
   Status Prefill(int layer, int q_pos0, int n, const float*, float* out) override {
     calls.push_back({AttentionCall::kPrefill, layer, q_pos0, n});

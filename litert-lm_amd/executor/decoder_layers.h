@@ -45,6 +45,11 @@ class SyntheticDecoderLayers : public DecoderLayers {
   Status ConsumeAttention(int layer, const float* attn) override;
   Status Logits(float* logits) override;
 
+  // Deterministic norm weights and rotary frequencies in the pattern of Gemma 3
+  // (query / key norm with a (1 + weight) scale, theta 10,000 on windowed layers
+  // and 1,000,000 on global ones) for tests of the fused step before attention.
+  static std::vector<LayerTransform> Transforms(const AttentionShape& shape);
+
   static uint32_t Mix(uint32_t x) {
     x ^= x >> 16;
     x *= 0x7feb352dU;

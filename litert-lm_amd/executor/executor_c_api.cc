@@ -34,6 +34,7 @@ struct hle_config {
   int32_t recording_backend;         // 1: no GPU, attention returns zeros and records calls
   int32_t execute_pending_on_single_id_chunk;
   float softcap;
+  int32_t pre_attention;             // 1: the layers hand over raw projections; Gemma-3-like norm + rotary constants
 };
 
 int hle_create(const hle_config* c, void** out, char** err) {
@@ -46,6 +47,7 @@ int hle_create(const hle_config* c, void** out, char** err) {
   shape.max_tokens = c->max_num_tokens;
   shape.softcap = c->softcap;
   if (c->layer_window) shape.layer_window.assign(c->layer_window, c->layer_window + c->num_layers);
+  if (c->pre_attention) shape.transforms = SyntheticDecoderLayers::Transforms(shape);
   auto settings = LlmExecutorSettings::CreateDefault(Backend::GPU_HIP);
   if (!settings.ok()) return Finish(settings.status(), err);
   settings->SetMaxNumTokens(c->max_num_tokens);

@@ -171,7 +171,12 @@ Status HipLlmExecutor::RunTokens(const std::vector<int32_t>& tokens, const std::
   RETURN_IF_ERROR(layers_->Begin(tokens, positions));
   for (int layer = 0; layer < shape.num_layers; ++layer) {
     RETURN_IF_ERROR(layers_->ProjectQkv(layer, q_.data(), k_.data(), v_.data()));
-    RETURN_IF_ERROR(backend_->Append(layer, pos0, n, k_.data(), v_.data()));
+    if (shape.transforms.empty()) {
+      RETURN_IF_ERROR(backend_->Append(layer, pos0, n, k_.data(), v_.data()));
+    } else {
+      // raw projections: norm + rotary embedding + cache write in one device pass
+      RETURN_IF_ERROR(backend_->PreAttention(layer, pos0, n, q_.data(), k_.data(), v_.data()));
+    }
     if (is_decode) {
       RETURN_IF_ERROR(backend_->Decode(layer, pos0 + 1, q_.data(), attn_.data()));
     } else {

@@ -5,6 +5,7 @@
 // (runtime/executor/llm_litert_compiled_model_executor.cc:528-533 hands out a
 // host-visible logits buffer right after the step).
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 #include "../../include/mi355_attn.h"
@@ -37,6 +38,23 @@ class Mi355AttentionBackend : public AttentionBackend {
       rc = mi355_attn_kv_append(h_, layer, 0, pos, n, k, v, &err);
     }
     return FromCode(rc, err, "kv_append");
+  }
+
+  Status PreAttention(int layer, int pos, int n, float* q, const float* k, const float* v) override {
+    char* err = nullptr;
+    const size_t qn = (size_t)n * shape_.num_q_heads * shape_.head_dim;
+    const size_t kn = (size_t)n * shape_.num_kv_heads * shape_.head_dim;
+    int rc;
+    if (fp16_) {
+      ToHalf(q, qn, &hq_);
+      ToHalf(k, kn, &ha_);
+      ToHalf(v, kn, &hb_);
+      rc = mi355_attn_pre_attention(h_, layer, 0, pos, n, hq_.data(), ha_.data(), hb_.data(), hq_.data(), &err);
+      if (rc == MI355_ATTN_OK) FromHalf(hq_, qn, q);
+    } else {
+      rc = mi355_attn_pre_attention(h_, layer, 0, pos, n, q, k, v, q, &err);
+    }
+    return FromCode(rc, err, "pre_attention");
   }
 
   Status Prefill(int layer, int q_pos0, int n, const float* q, float* out) override {
@@ -88,7 +106,7 @@ class Mi355AttentionBackend : public AttentionBackend {
   mi355_attn* h_;
   AttentionShape shape_;
   bool fp16_;
-  std::vector<_Float16> ha_, hb_;
+  std::vector<_Float16> ha_, hb_, hq_;
 };
 
 }  // namespace
@@ -115,6 +133,34 @@ StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const At
   char* err = nullptr;
   const int rc = mi355_attn_create(&cfg, &h, &err);
   if (rc != MI355_ATTN_OK) return FromCode(rc, err, "mi355_attn_create");
+  if (!shape.transforms.empty() && (int)shape.transforms.size() != shape.num_layers) {
+    mi355_attn_destroy(h);
+    return InvalidArgumentError("transforms needs one entry per layer.");
+  }
+  for (int layer = 0; layer < (int)shape.transforms.size(); ++layer) {
+    const LayerTransform& lt = shape.transforms[layer];
+    const size_t d = (size_t)shape.head_dim;
+    if ((!lt.q_weight.empty() && lt.q_weight.size() != d) || (!lt.k_weight.empty() && lt.k_weight.size() != d) ||
+        (!lt.rope_inv_freq.empty() && lt.rope_inv_freq.size() != d / 2)) {
+      mi355_attn_destroy(h);
+      return InvalidArgumentError("transform of layer " + std::to_string(layer) + ": wrong array length.");
+    }
+    mi355_attn_layer_transform t{};
+    t.struct_size = sizeof(t);
+    t.norm_q = lt.norm_q;
+    t.norm_k = lt.norm_k;
+    t.norm_v = lt.norm_v;
+    t.q_weight = lt.q_weight.empty() ? nullptr : lt.q_weight.data();
+    t.k_weight = lt.k_weight.empty() ? nullptr : lt.k_weight.data();
+    t.eps = lt.eps;
+    t.weight_offset = lt.weight_offset;
+    t.rope_inv_freq = lt.rope_inv_freq.empty() ? nullptr : lt.rope_inv_freq.data();
+    const int trc = mi355_attn_set_layer_transform(h, layer, &t, &err);
+    if (trc != MI355_ATTN_OK) {
+      mi355_attn_destroy(h);
+      return FromCode(trc, err, "mi355_attn_set_layer_transform");
+    }
+  }
   return std::unique_ptr<AttentionBackend>(new Mi355AttentionBackend(h, shape, fp16));
 }
 

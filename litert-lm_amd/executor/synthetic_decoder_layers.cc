@@ -4,6 +4,29 @@
 
 namespace litert::lm {
 
+std::vector<LayerTransform> SyntheticDecoderLayers::Transforms(const AttentionShape& shape) {
+  std::vector<LayerTransform> out(shape.num_layers);
+  const int d = shape.head_dim;
+  for (int layer = 0; layer < shape.num_layers; ++layer) {
+    LayerTransform& t = out[layer];
+    t.norm_q = t.norm_k = true;
+    t.eps = 1e-6f;
+    t.weight_offset = 1.f;
+    t.q_weight.resize(d);
+    t.k_weight.resize(d);
+    for (int c = 0; c < d; ++c) {
+      t.q_weight[c] = 0.25f * Unit((uint32_t)layer * 0x9E3779B1U + (uint32_t)c * 0x85EBCA77U + 9U);
+      t.k_weight[c] = 0.25f * Unit((uint32_t)layer * 0x9E3779B1U + (uint32_t)c * 0x85EBCA77U + 10U);
+    }
+    const bool local = !shape.layer_window.empty() && shape.layer_window[layer] > 0;
+    const double theta = local ? 10000.0 : 1000000.0;
+    t.rope_inv_freq.resize(d / 2);
+    for (int i = 0; i < d / 2; ++i)
+      t.rope_inv_freq[i] = static_cast<float>(1.0 / std::pow(theta, static_cast<double>(2 * i) / d));
+  }
+  return out;
+}
+
 Status SyntheticDecoderLayers::Begin(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions) {
   RET_CHECK_EQ(tokens.size(), positions.size());
   n_ = static_cast<int>(tokens.size());

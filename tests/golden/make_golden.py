@@ -11,6 +11,12 @@ in float64, stored as float32).
 
     python tests/golden/make_golden.py
 
+gemma3_pre_attention.npz holds the step before attention (per-head RMS norm with
+the (1 + weight) scale, rotary embedding) as the Gemma 3 building blocks of the
+`transformers` package compute it in float64 (Gemma3RMSNorm, apply_rotary_pos_emb,
+frequencies from Gemma3RotaryEmbedding.compute_default_rope_parameters): again
+an independent library, not the oracle it checks.
+
 softmax_kat.json is different in kind: the inputs and expected values that the
 reference's own test holds (runtime/components/sampling_cpu_util_test.cc:82-97),
 typed in as data.
@@ -76,8 +82,44 @@ def case(name, seed, hq, hkv, d, n_keys, q_pos, window=0, scale=None, softcap=0.
     print(name, out.shape, float(np.abs(out).max()))
 
 
+def gemma3_pre_attention():
+    from transformers.models.gemma3 import modeling_gemma3 as m
+
+    class Cfg:
+        head_dim = 256
+        hidden_size = 1024
+        num_attention_heads = 4
+        rope_parameters = {"sliding_attention": {"rope_theta": 10000.0}, "full_attention": {"rope_theta": 1000000.0}}
+
+    n, hq, hkv, d, pos0 = 24, 4, 1, 256, 3000
+    rng = np.random.default_rng(0xC0FFEE + 21)
+    q = exact(rng.standard_normal((n, hq, d), dtype=np.float32) * 2)
+    k = exact(rng.standard_normal((n, hkv, d), dtype=np.float32) * 2)
+    q_weight = exact((rng.standard_normal(d, dtype=np.float32) * 0.3))
+    k_weight = exact((rng.standard_normal(d, dtype=np.float32) * 0.3))
+    out = {"q": q, "k": k, "q_weight": q_weight, "k_weight": k_weight, "pos0": np.int32(pos0), "eps": np.float64(1e-6)}
+    for kind in ("sliding_attention", "full_attention"):
+        inv_freq, _ = m.Gemma3RotaryEmbedding.compute_default_rope_parameters(Cfg(), "cpu", layer_type=kind)
+        qn, kn = m.Gemma3RMSNorm(d, eps=1e-6).double(), m.Gemma3RMSNorm(d, eps=1e-6).double()
+        with torch.no_grad():
+            qn.weight.copy_(torch.from_numpy(q_weight).double())
+            kn.weight.copy_(torch.from_numpy(k_weight).double())
+            tq = qn(torch.from_numpy(q).double().permute(1, 0, 2)[None])
+            tk = kn(torch.from_numpy(k).double().permute(1, 0, 2)[None])
+            # the angle as the model forms it: float32 position times float32 frequency
+            ang = (torch.arange(pos0, pos0 + n, dtype=torch.float32)[:, None] * inv_freq.float()[None, :]).double()
+            emb = torch.cat([ang, ang], dim=-1)[None]
+            rq, rk = m.apply_rotary_pos_emb(tq, tk, emb.cos(), emb.sin())
+        out[f"inv_freq_{kind}"] = inv_freq.float().numpy()
+        out[f"q_out_{kind}"] = rq[0].permute(1, 0, 2).contiguous().numpy().astype(np.float32)
+        out[f"k_out_{kind}"] = rk[0].permute(1, 0, 2).contiguous().numpy().astype(np.float32)
+    np.savez_compressed(os.path.join(HERE, "gemma3_pre_attention.npz"), **out)
+    print("gemma3_pre_attention", out["q_out_full_attention"].shape, float(np.abs(out["q_out_full_attention"]).max()))
+
+
 def main():
     torch.set_num_threads(1)
+    gemma3_pre_attention()
     # decode rows (one query at the last position), shapes of configs 1 and 3 reduced in length
     case("decode_c1_like", 0xC0FFEE + 0, 4, 1, 256, 64, [63])
     case("decode_c3_like", 0xC0FFEE + 2, 8, 2, 256, 96, [95])

@@ -4,6 +4,7 @@ attention. Test helper only."""
 import numpy as np
 
 from oracle import attn_oracle as orc
+from oracle import pre_attention_oracle as po
 
 D = 256
 M32 = np.uint64(0xFFFFFFFF)
@@ -37,11 +38,20 @@ def key(*terms):
 
 
 class Twin:
-    def __init__(self, layers, hq, hkv, vocab, windows=None, softcap=0.0):
+    def __init__(self, layers, hq, hkv, vocab, windows=None, softcap=0.0, pre_attention=False):
         self.layers, self.hq, self.hkv, self.vocab = layers, hq, hkv, vocab
         self.windows = windows or [0] * layers
         self.softcap = softcap
         self.hidden = hq * D
+        self.pre_attention = pre_attention
+
+    def transform(self, layer):
+        """SyntheticDecoderLayers::Transforms: (q_weight, k_weight, inv_freq) of a layer."""
+        c = u(np.arange(D))
+        qw = np.float32(0.25) * unit(key(u(layer) * u(0x9E3779B1), c * u(0x85EBCA77), u(9)))
+        kw = np.float32(0.25) * unit(key(u(layer) * u(0x9E3779B1), c * u(0x85EBCA77), u(10)))
+        theta = 10000.0 if self.windows[layer] > 0 else 1000000.0
+        return qw, kw, po.rope_inv_freq(D, theta)
 
     def embed(self, tokens, positions):
         i = u(np.arange(self.hidden))[None, :]
@@ -94,6 +104,12 @@ class Twin:
         scale = D ** -0.5
         for layer in range(self.layers):
             q, k, v = self.project(layer, s)
+            if self.pre_attention:
+                if round_io is not None:  # the raw projections cross the boundary in the 16-bit type
+                    q, k, v = (x.astype(round_io).astype(np.float32) for x in (q, k, v))
+                qw, kw, inv_freq = self.transform(layer)
+                q, k, v = po.pre_attention(q, k, v, 0, q_weight=qw, k_weight=kw, norm_q=True, norm_k=True, eps=1e-6,
+                                           weight_offset=1.0, inv_freq=inv_freq)
             if round_io is not None:
                 q, k, v = (x.astype(round_io).astype(np.float32) for x in (q, k, v))
             attn = orc.sdpa(q, k, v, scale, window=self.windows[layer], softcap=self.softcap)

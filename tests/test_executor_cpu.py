@@ -130,3 +130,12 @@ def test_error_paths():
     with pytest.raises(X.ExecutorError) as e:
         X.HipLlmExecutor(2, 4, 1, 16, 0, recording_backend=True)
     assert e.value.code == INVALID_ARGUMENT
+
+
+def test_fused_step_before_attention_keeps_the_step_logic():
+    # raw projections + norm / rotary constants per layer: same chunks, positions and steps
+    with make(runners=(4,), pre_attention=True) as ex, make(runners=(4,)) as plain:
+        for e in (ex, plain):
+            e.prefill([10, 11, 12, 13, 14, 15, 16])
+            e.decode()
+        assert ex.runs() == plain.runs() and ex.current_step() == plain.current_step() == 8

@@ -15,7 +15,7 @@ from oracle import attn_oracle as orc  # noqa: E402
 from oracle import c_oracle  # noqa: E402
 
 GOLDEN = os.path.join(ROOT, "tests", "golden")
-CASES = sorted(glob.glob(os.path.join(GOLDEN, "*.npz")))
+CASES = sorted(glob.glob(os.path.join(GOLDEN, "decode_*.npz")) + glob.glob(os.path.join(GOLDEN, "prefill_*.npz")))
 
 
 def load(path):

@@ -25,15 +25,19 @@ def rel(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
+@pytest.mark.parametrize("pre_attention", [False, True])
 @pytest.mark.parametrize("fp16", [False, True])
-def test_prefill_chunks_then_greedy_decode_match_whole_sequence_reference(fp16):
+def test_prefill_chunks_then_greedy_decode_match_whole_sequence_reference(fp16, pre_attention):
+    # pre_attention: the layers hand over raw projections and the fused device step
+    # (RMS norm + rotary embedding + cache write) runs before every attention call
     layers, hq, hkv, vocab = 3, 4, 1, 48
     windows = [0, 24, 0]
     rng = np.random.default_rng(11)
     prompt = [int(x) for x in rng.integers(0, vocab, size=71)]
     tol = 2e-3 if fp16 else 2e-5
-    twin = Twin(layers, hq, hkv, vocab, windows)
-    with X.HipLlmExecutor(layers, hq, hkv, vocab, 256, runner_lengths=(32, 8), layer_window=windows, fp16=fp16) as ex:
+    twin = Twin(layers, hq, hkv, vocab, windows, pre_attention=pre_attention)
+    with X.HipLlmExecutor(layers, hq, hkv, vocab, 256, runner_lengths=(32, 8), layer_window=windows, fp16=fp16,
+                          pre_attention=pre_attention) as ex:
         assert "MI355X" in ex.backend_name()
         ex.prefill(prompt[:40])   # chunks of 32 and 8, last id deferred
         ex.prefill(prompt[40:])   # pending id goes first
@@ -43,7 +47,7 @@ def test_prefill_chunks_then_greedy_decode_match_whole_sequence_reference(fp16):
             logits = ex.decode_logits()  # executes the pending token at position len(seq)-1
             ref = twin.forward_all(seq, round_io=np.float16 if fp16 else None)[-1]
             err = rel(logits, ref)
-            print(f"fp16={fp16} step {step}: logits rel_err {err:.2e}", flush=True)
+            print(f"fp16={fp16} pre_attention={pre_attention} step {step}: logits rel_err {err:.2e}", flush=True)
             assert err < tol
             assert int(np.argmax(logits)) == int(np.argmax(ref))
             nxt = int(np.argmax(logits))

@@ -404,7 +404,8 @@ def test_c5_int8_full_size_properties():
 
 # ------------------------------------------------------------------ error behaviour (no kernel is launched)
 # ------------------------------------------------------------------ golden vectors
-GOLDEN = sorted(__import__("glob").glob(os.path.join(ROOT, "tests", "golden", "*.npz")))
+GOLDEN = sorted(__import__("glob").glob(os.path.join(ROOT, "tests", "golden", "decode_*.npz")) +
+                __import__("glob").glob(os.path.join(ROOT, "tests", "golden", "prefill_*.npz")))
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
