@@ -247,6 +247,31 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   vec8 p_prev[NP], p_cur[NP];  // probabilities of the previous block / of this one
   float bm, alpha, neg_m, lsum;
 
+  // The visibility test rides on the accumulator the scores of a block are summed
+  // into: 0 where the key is visible, -inf where not. Blocks in the middle of the
+  // causal triangle (every key visible to every row of the wave) start from plain
+  // zeros, so only the block on the diagonal and the one at the window's edge pay
+  // for the 16 comparisons. With a soft cap the test follows the cap instead.
+  const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
+  auto koff_of = [](int e) { return 16 * ((e >> 2) & 1) + 8 * (e >> 3) + (e & 3); };  // key_of_row(8*(e>>2) + 4*hh + (e&3)) - 4*hh
+  auto all_visible = [&](int blk) {
+    const int key0 = (kb_lo + blk) * kKeysPerBlock;
+    return CAP || (key0 + kKeysPerBlock - 1 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim);
+  };
+  // the first MFMA of a block's scores, on zeros or on the 0 / -inf tile
+  auto first_scores = [&](vec8 k_op, vec8 q_op, int blk) {
+    f16v init;
+    if (all_visible(blk)) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) init[e] = 0.f;
+      return E::mfma(k_op, q_op, init);
+    }
+    const int d0 = my_pos - (kb_lo + blk) * kKeysPerBlock - 4 * hh;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) init[e] = (unsigned)(d0 - koff_of(e)) < wlim ? 0.f : -INFINITY;
+    return E::mfma(k_op, q_op, init);
+  };
+
   // One pipeline step: the vector ALU turns the scores of block i (in sa) into
   // probabilities while the matrix core multiplies the probabilities of block
   // i-1 into the accumulators (PREV) and computes the scores of block i+1
@@ -254,12 +279,10 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   // the LDS read of an operand a few MFMAs ahead and a slice of the softmax,
   // and the compiler may not move code across chunk borders, so the three
   // instruction streams stay dealt out evenly. The softmax is a list of 34
-  // pieces: 16 x (soft cap, visibility test, running max of one score), the
+  // pieces: 16 x (soft cap and its visibility test if any, running max of one score), the
   // exchange of the max between the two lanes of a query (2 pieces, the LDS
   // crossbar has latency), 16 x (exp2, sum, conversion of one score).
-  // The visibility test is applied to every block, also those in the middle of
-  // the causal triangle: it hides under the MFMAs, and a single variant of the
-  // loop body keeps the accumulators in place.
+  // A single variant of the loop body keeps the accumulators in place.
   auto step = [&](int i, bool fetch_k, bool fetch_v, auto has_prev, auto has_next) {
     constexpr bool PREV = decltype(has_prev)::value, NEXT = decltype(has_next)::value;
     constexpr int GP = PREV ? NDP * NP : 0;  // chunks with a P.V MFMA
@@ -276,10 +299,12 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
       if constexpr (P < 16) {
         constexpr int e = P;
         float x = sa[e];
-        if constexpr (CAP) x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
-        constexpr int koff = 16 * ((e >> 2) & 1) + 8 * (e >> 3) + (e & 3);  // key_of_row(8*(e>>2) + 4*hh + (e&3)) - 4*hh
-        x = (unsigned)(dist0 - koff) < wlim ? x : -INFINITY;
-        sa[e] = x;
+        if constexpr (CAP) {
+          // (the cap maps -inf to -cap, so here the test cannot ride on the accumulator)
+          x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
+          x = (unsigned)(dist0 - koff_of(e)) < wlim ? x : -INFINITY;
+          sa[e] = x;
+        }
         bm = e == 0 ? x : fmaxf(bm, x);
       } else if constexpr (P == 16) {
         lsum = __shfl_xor(bm, 32, 64);  // (lsum is free until the sums start)
@@ -326,10 +351,6 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
 #pragma unroll
       for (int j = 0; j < kAhead; ++j) kk[j] = *reinterpret_cast<const vec8*>(kb + j * 512);
     }
-    if constexpr (NEXT) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) na[e] = 0.f;
-    }
     // The transfers of K(i+3) and V(i+1) are requested one at a time, spread
     // over the step: issued back to back by all four waves they would queue
     // up in the CU's one vector-memory pipeline and stall the waves in front
@@ -358,7 +379,8 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
           kk[g - (GP - kAhead)] = *reinterpret_cast<const vec8*>(kb + (g - (GP - kAhead)) * 512);
       } else if constexpr (g < GP + GQ) {
         constexpr int j = g - GP;
-        na = E::mfma(kk[j % kAhead], q0[j], na);
+        if constexpr (j == 0) na = first_scores(kk[0], q0[0], i + 1);
+        else na = E::mfma(kk[j % kAhead], q0[j], na);
         if constexpr (j + kAhead < NJ) kk[j % kAhead] = *reinterpret_cast<const vec8*>(kb + (j + kAhead) * 512);
       }
       static_for<kPieces>([&](auto pc) {
@@ -379,12 +401,11 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     const uint8_t* kb = sm_k + k_off;
 #pragma unroll
     for (int j = 0; j < kAhead; ++j) kk[j] = *reinterpret_cast<const vec8*>(kb + j * 512);
-#pragma unroll
-    for (int e = 0; e < 16; ++e) sa[e] = 0.f;
     static_for<NJ>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
       __builtin_amdgcn_sched_barrier(0);
-      sa = E::mfma(kk[j % kAhead], q0[j], sa);
+      if constexpr (j == 0) sa = first_scores(kk[0], q0[0], 0);
+      else sa = E::mfma(kk[j % kAhead], q0[j], sa);
       if constexpr (j + kAhead < NJ) kk[j % kAhead] = *reinterpret_cast<const vec8*>(kb + (j + kAhead) * 512);
     });
     __builtin_amdgcn_sched_barrier(0);
