@@ -33,6 +33,11 @@ class _Config(ctypes.Structure):
     ]
 
 
+class LoopResult(ctypes.Structure):
+    _fields_ = [("last_prefill_id", ctypes.c_int32), ("n_tokens", ctypes.c_int32),
+                ("cache_full_error", ctypes.c_int32), ("current_step", ctypes.c_int32)]
+
+
 def lib():
     global _lib
     if _lib is None:
@@ -57,6 +62,23 @@ def lib():
         L.hle_get_run.argtypes = [vp, i32, i32p, i32p, i32p, i32]
         L.hle_backend_from_string.argtypes = [ctypes.c_char_p]
         L.hle_plan.argtypes = [i32p, i32, i32, i32p, i32p, i32]
+        L.hle_bi_create.argtypes = [i32, i32]
+        L.hle_bi_create.restype = vp
+        L.hle_bi_destroy.argtypes = [vp]
+        L.hle_bi_destroy.restype = None
+        L.hle_bi_call.argtypes = [vp, i32, ctypes.c_char_p, ctypes.c_uint64, errp]
+        L.hle_bi_count.argtypes = [vp, i32]
+        L.hle_bi_value.argtypes = [vp, i32, ctypes.c_char_p, i32]
+        L.hle_bi_value.restype = ctypes.c_double
+        L.hle_bi_report.argtypes = [vp]
+        L.hle_bi_report.restype = vp
+        L.hle_format_duration.argtypes = [ctypes.c_int64]
+        L.hle_format_duration.restype = vp
+        L.hle_stop_detector_run.argtypes = [i32, i32p, i32p, i32, i32p, i32, i32p, i32p, i32, i32p]
+        resp = ctypes.POINTER(LoopResult)
+        L.hle_fake_loop.argtypes = [i32p, i32, i32, i32p, i32, i32p, i32, i32, i32p, i32, i32, i32, i32, i32, i32p, i32,
+                                    resp, errp, errp]
+        L.hle_run_benchmark.argtypes = [vp, i32p, i32, i32, i32, i32p, i32, resp, errp, errp]
         _lib = L
     return _lib
 
@@ -155,6 +177,108 @@ class HipLlmExecutor:
             n = lib().hle_get_run(self._h, i, ctypes.byref(dec), toks, pos, cap)
             out.append(("decode" if dec.value else "prefill", list(toks[:n]), list(pos[:n])))
         return out
+
+
+def _take_text(ptr) -> str:
+    if not ptr:
+        return ""
+    text = ctypes.string_at(ptr).decode("utf-8", "replace")
+    _attn._libc.free(ptr)
+    return text
+
+
+class BenchmarkInfo:
+    """The C++ BenchmarkInfo (executor/benchmark_info.h) behind its test surface."""
+    INIT_START, INIT_END, PREFILL_START, PREFILL_END, DECODE_START, DECODE_END, MARK = range(7)
+
+    def __init__(self, num_prefill_tokens=0, num_decode_tokens=0):
+        self._h = ctypes.c_void_p(lib().hle_bi_create(num_prefill_tokens, num_decode_tokens))
+
+    def __del__(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            lib().hle_bi_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def _call(self, what, name=b"", tokens=0):
+        err = ctypes.c_void_p()
+        _check(lib().hle_bi_call(self._h, what, name.encode() if isinstance(name, str) else name, tokens,
+                                 ctypes.byref(err)), err)
+
+    def time_init_phase_start(self, name): self._call(self.INIT_START, name)
+    def time_init_phase_end(self, name): self._call(self.INIT_END, name)
+    def time_prefill_turn_start(self): self._call(self.PREFILL_START)
+    def time_prefill_turn_end(self, tokens): self._call(self.PREFILL_END, tokens=tokens)
+    def time_decode_turn_start(self): self._call(self.DECODE_START)
+    def time_decode_turn_end(self, tokens): self._call(self.DECODE_END, tokens=tokens)
+    def time_mark_delta(self, name): self._call(self.MARK, name)
+
+    def num_init_phases(self): return lib().hle_bi_count(self._h, 0)
+    def total_prefill_turns(self): return lib().hle_bi_count(self._h, 1)
+    def total_decode_turns(self): return lib().hle_bi_count(self._h, 2)
+    def num_marks(self): return lib().hle_bi_count(self._h, 3)
+    def init_phase_seconds(self, name): return lib().hle_bi_value(self._h, 0, name.encode(), 0)
+    def mark_seconds(self, name): return lib().hle_bi_value(self._h, 3, name.encode(), 0)
+    def prefill_tokens_per_sec(self, i): return lib().hle_bi_value(self._h, 1, b"", i)
+    def decode_tokens_per_sec(self, i): return lib().hle_bi_value(self._h, 2, b"", i)
+
+    def report(self) -> str:
+        return _take_text(lib().hle_bi_report(self._h))
+
+
+def format_duration(ns: int) -> str:
+    return _take_text(lib().hle_format_duration(int(ns)))
+
+
+def stop_detector_run(batch, sequences, tokens, reset=False):
+    """tokens: [steps][batch]. Returns (step at which every item had stopped, add status codes,
+    steps-before-stop per item, all-done after the optional reset)."""
+    flat = [t for seq in sequences for t in seq]
+    lens = [len(seq) for seq in sequences]
+    steps = len(tokens)
+    toks = [t for row in tokens for t in row]
+    codes = (ctypes.c_int32 * max(1, len(sequences)))()
+    before = (ctypes.c_int32 * batch)()
+    done = ctypes.c_int32(-1)
+    i = lib().hle_stop_detector_run(batch, _arr(flat) if flat else None, _arr(lens) if lens else None, len(sequences),
+                                    _arr(toks) if toks else None, steps, codes, before, int(reset), ctypes.byref(done))
+    if i < 0:
+        raise ExecutorError(-i, "ProcessTokens")
+    return i, list(codes[:len(sequences)]), list(before), (None if not reset else bool(done.value))
+
+
+def _loop_outputs(rc, err, out, res, report):
+    text = _take_text(report.value)
+    _check(rc, err)
+    return {"tokens": list(out[:res.n_tokens]), "last_prefill_id": res.last_prefill_id,
+            "cache_full_error": bool(res.cache_full_error), "current_step": res.current_step, "report": text}
+
+
+def fake_loop(prompt, expected_prefill, decode_script, *, bos=2, max_num_tokens=0, stop_sequence=(), bench_prefill=0,
+              bench_decode=0, streaming=False, do_prefill=True):
+    """Prefill + decode loop of executor/pipeline.h over the scripted FakeLlmExecutor."""
+    cap = 4096
+    out = (ctypes.c_int32 * cap)()
+    res = LoopResult()
+    err, report = ctypes.c_void_p(), ctypes.c_void_p()
+    stop = list(stop_sequence)
+    rc = lib().hle_fake_loop(_arr(prompt) if prompt else None, len(prompt), bos,
+                             _arr(expected_prefill) if expected_prefill else None, len(expected_prefill),
+                             _arr(decode_script) if decode_script else None, len(decode_script), max_num_tokens,
+                             _arr(stop) if stop else None, len(stop), bench_prefill, bench_decode, int(streaming),
+                             int(do_prefill), out, cap, ctypes.byref(res), ctypes.byref(report), ctypes.byref(err))
+    return _loop_outputs(rc, err, out, res, report)
+
+
+def run_benchmark(executor: "HipLlmExecutor", prompt, bench_prefill, bench_decode):
+    """The reference's benchmark protocol (prefill turn of `bench_prefill` ids, `bench_decode` decode
+    steps) on a HipLlmExecutor; returns the ids, the step counter and the BenchmarkInfo text."""
+    cap = max(16, bench_decode + 16)
+    out = (ctypes.c_int32 * cap)()
+    res = LoopResult()
+    err, report = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = lib().hle_run_benchmark(executor._h, _arr(prompt) if prompt else None, len(prompt), bench_prefill, bench_decode,
+                                 out, cap, ctypes.byref(res), ctypes.byref(report), ctypes.byref(err))
+    return _loop_outputs(rc, err, out, res, report)
 
 
 def backend_from_string(s: str) -> int:

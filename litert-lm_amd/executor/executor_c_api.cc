@@ -6,7 +6,13 @@
 #include <cstring>
 #include <memory>
 
+#include <sstream>
+
+#include "benchmark_info.h"
+#include "fake_llm_executor.h"
 #include "hip_llm_executor.h"
+#include "pipeline.h"
+#include "stop_token_detector.h"
 
 using namespace litert::lm;
 
@@ -20,6 +26,11 @@ int Finish(const Status& s, char** err) {
 }
 ExecutorInputs IdsInput(const int32_t* ids, int batch, int n) {
   return ExecutorInputs(ExecutorTextData(TensorBuffer::CopyFrom(ElementType::kInt32, {batch, n}, ids)));
+}
+char* CopyText(const std::string& text) {
+  char* out = static_cast<char*>(malloc(text.size() + 1));
+  if (out) memcpy(out, text.c_str(), text.size() + 1);
+  return out;
 }
 }  // namespace
 
@@ -131,6 +142,158 @@ int hle_plan(const int32_t* runner_lengths, int num_runners, int n, int32_t* len
     ++k;
   }
   return k;
+}
+
+// ---- BenchmarkInfo, stop-token detector and the prefill / decode loop (test surface)
+
+void* hle_bi_create(int32_t num_prefill_tokens, int32_t num_decode_tokens) {
+  BenchmarkParams p;
+  p.num_prefill_tokens = num_prefill_tokens;
+  p.num_decode_tokens = num_decode_tokens;
+  return new BenchmarkInfo(p);
+}
+void hle_bi_destroy(void* bi) { delete static_cast<BenchmarkInfo*>(bi); }
+
+// what: 0/1 init phase start/end, 2/3 prefill turn start/end, 4/5 decode turn start/end, 6 mark
+int hle_bi_call(void* bi, int32_t what, const char* name, uint64_t tokens, char** err) {
+  auto* b = static_cast<BenchmarkInfo*>(bi);
+  switch (what) {
+    case 0: return Finish(b->TimeInitPhaseStart(name), err);
+    case 1: return Finish(b->TimeInitPhaseEnd(name), err);
+    case 2: return Finish(b->TimePrefillTurnStart(), err);
+    case 3: return Finish(b->TimePrefillTurnEnd(tokens), err);
+    case 4: return Finish(b->TimeDecodeTurnStart(), err);
+    case 5: return Finish(b->TimeDecodeTurnEnd(tokens), err);
+    case 6: return Finish(b->TimeMarkDelta(name), err);
+    default: return Finish(InvalidArgumentError("unknown call"), err);
+  }
+}
+// what: 0 init phases, 1 prefill turns, 2 decode turns, 3 marks
+int hle_bi_count(void* bi, int32_t what) {
+  auto* b = static_cast<BenchmarkInfo*>(bi);
+  switch (what) {
+    case 0: return static_cast<int>(b->GetInitPhases().size());
+    case 1: return static_cast<int>(b->GetTotalPrefillTurns());
+    case 2: return static_cast<int>(b->GetTotalDecodeTurns());
+    default: return static_cast<int>(b->GetMarkDurations().size());
+  }
+}
+// Seconds of an init phase (what 0) or mark (what 3) by name, tokens per second of a prefill (1) / decode (2) turn by index; -1 if absent.
+double hle_bi_value(void* bi, int32_t what, const char* name, int32_t index) {
+  auto* b = static_cast<BenchmarkInfo*>(bi);
+  if (what == 1) return b->GetPrefillTokensPerSec(index);
+  if (what == 2) return b->GetDecodeTokensPerSec(index);
+  const auto& m = what == 0 ? b->GetInitPhases() : b->GetMarkDurations();
+  auto it = m.find(name);
+  return it == m.end() ? -1.0 : static_cast<double>(it->second.count()) * 1e-9;
+}
+char* hle_bi_report(void* bi) {
+  std::ostringstream os;
+  os << *static_cast<BenchmarkInfo*>(bi);
+  return CopyText(os.str());
+}
+char* hle_format_duration(int64_t ns) { return CopyText(FormatDuration(Duration(ns))); }
+
+// Feeds tokens [steps][batch] step by step until every item has stopped; returns the index of that step (steps if
+// never). add_codes[n_seqs] receives the status of each AddStopTokenSequence, steps_before[batch] the detector's
+// count per item; reset != 0 calls ResetBatch() at the end and reports AllDone after it in *done_after_reset.
+int hle_stop_detector_run(int32_t batch, const int32_t* seqs_flat, const int32_t* seq_lens, int32_t n_seqs,
+                          const int32_t* tokens, int32_t steps, int32_t* add_codes, int32_t* steps_before,
+                          int32_t reset, int32_t* done_after_reset) {
+  StopTokenDetector detector(batch);
+  const int32_t* p = seqs_flat;
+  for (int i = 0; i < n_seqs; ++i) {
+    add_codes[i] = static_cast<int>(detector.AddStopTokenSequence(std::vector<int>(p, p + seq_lens[i])).code());
+    p += seq_lens[i];
+  }
+  int i = 0;
+  for (; i < steps; ++i) {
+    Status s = detector.ProcessTokens(tokens + (size_t)i * batch, batch);
+    if (!s.ok()) return -static_cast<int>(s.code());
+    if (*detector.AllDone()) break;
+  }
+  if (reset) {
+    detector.ResetBatch();
+    *done_after_reset = *detector.AllDone() ? 1 : 0;
+  }
+  for (int b = 0; b < batch; ++b) steps_before[b] = detector.GetStepsBeforeStopTokens()[b];
+  return i;
+}
+
+struct hle_loop_result {
+  int32_t last_prefill_id;
+  int32_t n_tokens;          // ids produced by the decode loop
+  int32_t cache_full_error;  // the streaming observer saw "Maximum kv-cache size reached."
+  int32_t current_step;
+};
+
+namespace {
+int RunLoop(LlmExecutor& ex, const int32_t* prompt, int n_prompt, int bos, const int32_t* stop_seq, int n_stop,
+            int bench_prefill, int bench_decode, int streaming, int do_prefill, int32_t* out_tokens, int cap,
+            hle_loop_result* res, char** report, char** err) {
+  std::optional<BenchmarkInfo> info;
+  if (bench_prefill > 0 || bench_decode > 0) {
+    BenchmarkParams p;
+    p.num_prefill_tokens = bench_prefill;
+    p.num_decode_tokens = bench_decode;
+    info.emplace(p);
+  }
+  *res = hle_loop_result{-1, 0, 0, 0};
+  if (do_prefill) {
+    auto last = Prefill(ex, std::vector<int>(prompt, prompt + n_prompt), bos, /*wait_for_completion=*/true, info);
+    if (!last.ok()) return Finish(last.status(), err);
+    res->last_prefill_id = *last;
+  }
+  StopTokenDetector detector(1);
+  if (n_stop > 0) {
+    Status s = detector.AddStopTokenSequence(std::vector<int>(stop_seq, stop_seq + n_stop));
+    if (!s.ok()) return Finish(s, err);
+  }
+  std::vector<int> tokens;
+  if (streaming) {
+    Status s = DecodeStreaming(
+        ex, detector, info, [&](int id) { tokens.push_back(id); },
+        [&](const Status& e) { res->cache_full_error |= e.message() == "Maximum kv-cache size reached." ? 1 : 0; });
+    if (!s.ok()) return Finish(s, err);
+  } else {
+    auto r = Decode(ex, detector, info);
+    if (!r.ok()) return Finish(r.status(), err);
+    tokens = *r;
+  }
+  res->n_tokens = static_cast<int>(tokens.size());
+  for (int i = 0; i < res->n_tokens && i < cap; ++i) out_tokens[i] = tokens[i];
+  res->current_step = *ex.GetCurrentStep();
+  if (report && info.has_value()) {
+    std::ostringstream os;
+    os << *info;
+    *report = CopyText(os.str());
+  }
+  return 0;
+}
+}  // namespace
+
+// The loop over a scripted executor: expected_prefill (n_expected ids) is what Prefill must receive,
+// decode_script the ids Decode hands out; max_num_tokens 0 keeps the fake's 1024.
+int hle_fake_loop(const int32_t* prompt, int32_t n_prompt, int32_t bos, const int32_t* expected_prefill,
+                  int32_t n_expected, const int32_t* decode_script, int32_t n_decode, int32_t max_num_tokens,
+                  const int32_t* stop_seq, int32_t n_stop, int32_t bench_prefill, int32_t bench_decode,
+                  int32_t streaming, int32_t do_prefill, int32_t* out_tokens, int32_t cap, hle_loop_result* res,
+                  char** report, char** err) {
+  std::vector<std::vector<int>> decode_set;
+  for (int i = 0; i < n_decode; ++i) decode_set.push_back({decode_script[i]});
+  FakeLlmExecutor ex(/*vocab_size=*/2560, {std::vector<int>(expected_prefill, expected_prefill + n_expected)}, decode_set);
+  if (max_num_tokens > 0) ex.GetMutableExecutorSettings()->SetMaxNumTokens(max_num_tokens);
+  return RunLoop(ex, prompt, n_prompt, bos, stop_seq, n_stop, bench_prefill, bench_decode, streaming, do_prefill,
+                 out_tokens, cap, res, report, err);
+}
+
+// The reference's benchmark protocol on a HipLlmExecutor: one prefill turn of bench_prefill ids, then
+// bench_decode decode steps; *report receives the BenchmarkInfo text (malloc'd).
+int hle_run_benchmark(void* h, const int32_t* prompt, int32_t n_prompt, int32_t bench_prefill, int32_t bench_decode,
+                      int32_t* out_tokens, int32_t cap, hle_loop_result* res, char** report, char** err) {
+  const int32_t never = -1;  // a stop sequence no id matches: the step counts of the benchmark end the loop
+  return RunLoop(*static_cast<HipLlmExecutor*>(h), prompt, n_prompt, /*bos=*/2, &never, 1, bench_prefill, bench_decode,
+                 /*streaming=*/0, /*do_prefill=*/1, out_tokens, cap, res, report, err);
 }
 
 }  // extern "C"

@@ -18,6 +18,7 @@ enum class StatusCode : int {
   kOk = 0,
   kInvalidArgument = 3,
   kNotFound = 5,
+  kAlreadyExists = 6,
   kResourceExhausted = 8,
   kFailedPrecondition = 9,
   kOutOfRange = 11,
@@ -44,6 +45,7 @@ inline Status InvalidArgumentError(std::string m) { return Status(StatusCode::kI
 inline Status InternalError(std::string m) { return Status(StatusCode::kInternal, std::move(m)); }
 inline Status UnimplementedError(std::string m) { return Status(StatusCode::kUnimplemented, std::move(m)); }
 inline Status FailedPreconditionError(std::string m) { return Status(StatusCode::kFailedPrecondition, std::move(m)); }
+inline Status AlreadyExistsError(std::string m) { return Status(StatusCode::kAlreadyExists, std::move(m)); }
 inline Status NotFoundError(std::string m) { return Status(StatusCode::kNotFound, std::move(m)); }
 inline Status OutOfRangeError(std::string m) { return Status(StatusCode::kOutOfRange, std::move(m)); }
 

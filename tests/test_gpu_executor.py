@@ -68,3 +68,25 @@ def test_prefill_chunks_then_greedy_decode_match_whole_sequence_reference(fp16, 
         t2 = ex.decode()
         ref = twin.forward_all(prompt[:10] + [t1], round_io=np.float16 if fp16 else None)[-1]
         assert t2 == int(np.argmax(ref))
+
+
+def test_readme_benchmark_protocol_in_the_reference_report_format():
+    """`litert_lm_main --benchmark --benchmark_prefill_tokens=1024 --benchmark_decode_tokens=256`
+    (README.md:390-400 of the reference) on the HIP executor: Gemma-3-like attention stack
+    (26 layers, 5 local : 1 global, window 512, Hq4 / Hkv1, fp16), synthetic layers around it."""
+    import re
+    layers, hq, hkv, vocab = 26, 4, 1, 64
+    windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
+    with X.HipLlmExecutor(layers, hq, hkv, vocab, 2048, runner_lengths=(1024,), layer_window=windows, fp16=True,
+                          pre_attention=True) as ex:
+        r = X.run_benchmark(ex, [3, 1, 4, 1, 5, 9, 2, 6], 1024, 256)
+        print(r["report"], flush=True)
+        assert len(r["tokens"]) == 256 and r["current_step"] == 1024 + 256
+        assert all(0 <= t < vocab for t in r["tokens"])
+        runs = ex.runs()
+        assert [len(t) for k, t, _ in runs if k == "prefill"] == [1023]   # the 1024th id is the first decode step
+        assert sum(1 for k, _, _ in runs if k == "decode") == 256
+        assert re.search(r"Prefill Turn 1: Processed 1024 tokens in \S+ duration\.\n      Prefill Speed: \d+\.\d\d tokens/sec\.",
+                         r["report"])
+        assert re.search(r"Decode Turn 1: Processed 256 tokens in \S+ duration\.\n      Decode Speed: \d+\.\d\d tokens/sec\.",
+                         r["report"])
