@@ -79,6 +79,8 @@ def lib():
         L.hle_fake_loop.argtypes = [i32p, i32, i32, i32p, i32, i32p, i32, i32, i32p, i32, i32, i32, i32, i32, i32p, i32,
                                     resp, errp, errp]
         L.hle_run_benchmark.argtypes = [vp, i32p, i32, i32, i32, i32p, i32, resp, errp, errp]
+        L.hle_litertlm_header.argtypes = [ctypes.c_char_p, vp, ctypes.c_uint64, errp, errp]
+        L.hle_litertlm_read.argtypes = [ctypes.c_char_p, i32, i32, i32, errp, ctypes.POINTER(ctypes.c_uint64), errp]
         _lib = L
     return _lib
 
@@ -279,6 +281,48 @@ def run_benchmark(executor: "HipLlmExecutor", prompt, bench_prefill, bench_decod
     rc = lib().hle_run_benchmark(executor._h, _arr(prompt) if prompt else None, len(prompt), bench_prefill, bench_decode,
                                  out, cap, ctypes.byref(res), ctypes.byref(report), ctypes.byref(err))
     return _loop_outputs(rc, err, out, res, report)
+
+
+# AnySectionDataType of the .litertlm container
+SECTION_NONE, SECTION_BINARY, SECTION_DEPRECATED, SECTION_TFLITE, SECTION_SP_TOKENIZER, SECTION_LLM_METADATA, \
+    SECTION_HF_TOKENIZER_ZLIB = range(7)
+
+
+def litertlm_header(path=None, data=None) -> dict:
+    """Header of a .litertlm file (or of a bytes object): version, system metadata, section map."""
+    import json
+    text, err = ctypes.c_void_p(), ctypes.c_void_p()
+    if path is not None:
+        rc = lib().hle_litertlm_header(str(path).encode(), None, 0, ctypes.byref(text), ctypes.byref(err))
+    else:
+        buf = ctypes.create_string_buffer(bytes(data), len(data))
+        rc = lib().hle_litertlm_header(None, ctypes.cast(buf, ctypes.c_void_p), len(data), ctypes.byref(text),
+                                       ctypes.byref(err))
+    out = _take_text(text.value)
+    _check(rc, err)
+    return json.loads(out)
+
+
+def _litertlm_read(path, what, idx=0, expected_type=0) -> bytes:
+    data, err, n = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_uint64()
+    rc = lib().hle_litertlm_read(str(path).encode(), what, idx, expected_type, ctypes.byref(data), ctypes.byref(n),
+                                 ctypes.byref(err))
+    _check(rc, err)
+    out = ctypes.string_at(data.value, n.value)
+    _attn._libc.free(data.value)
+    return out
+
+
+def litertlm_section(path, idx, expected_type) -> bytes:
+    return _litertlm_read(path, 0, idx, expected_type)
+
+
+def litertlm_hf_tokenizer_json(path, idx=None) -> bytes:
+    return _litertlm_read(path, 2) if idx is None else _litertlm_read(path, 1, idx)
+
+
+def litertlm_any_binary(path) -> bytes:
+    return _litertlm_read(path, 3)
 
 
 def backend_from_string(s: str) -> int:

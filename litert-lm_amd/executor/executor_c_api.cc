@@ -11,6 +11,7 @@
 #include "benchmark_info.h"
 #include "fake_llm_executor.h"
 #include "hip_llm_executor.h"
+#include "litertlm_reader.h"
 #include "pipeline.h"
 #include "stop_token_detector.h"
 
@@ -294,6 +295,86 @@ int hle_run_benchmark(void* h, const int32_t* prompt, int32_t n_prompt, int32_t 
   const int32_t never = -1;  // a stop sequence no id matches: the step counts of the benchmark end the loop
   return RunLoop(*static_cast<HipLlmExecutor*>(h), prompt, n_prompt, /*bos=*/2, &never, 1, bench_prefill, bench_decode,
                  /*streaming=*/0, /*do_prefill=*/1, out_tokens, cap, res, report, err);
+}
+
+}  // extern "C"
+
+// ---- .litertlm container reader (test surface)
+
+namespace {
+std::string JsonString(const std::string& text) {
+  std::string out = "\"";
+  for (unsigned char c : text) {
+    if (c == '"' || c == '\\') {
+      out.push_back('\\');
+      out.push_back(static_cast<char>(c));
+    } else if (c < 0x20) {
+      char buf[8];
+      snprintf(buf, sizeof(buf), "\\u%04x", c);
+      out += buf;
+    } else {
+      out.push_back(static_cast<char>(c));
+    }
+  }
+  return out + "\"";
+}
+std::string JsonItems(const std::vector<schema::KeyValue>& items) {
+  std::string out = "[";
+  for (size_t i = 0; i < items.size(); ++i) {
+    const schema::KeyValue& kv = items[i];
+    out += std::string(i ? ", " : "") + "{\"key\": " + JsonString(kv.key) + ", \"type\": " + std::to_string(kv.type) +
+           ", \"value\": " + JsonString(kv.ToString()) + "}";
+  }
+  return out + "]";
+}
+std::string DescribeHeader(const schema::LitertlmHeader& h) {
+  std::string out = "{\"version\": [" + std::to_string(h.major_version) + ", " + std::to_string(h.minor_version) + ", " +
+                    std::to_string(h.patch_version) + "], \"header_end_offset\": " + std::to_string(h.header_end_offset) +
+                    ", \"system_metadata\": " + JsonItems(h.system_metadata) + ", \"sections\": [";
+  for (size_t i = 0; i < h.sections.size(); ++i) {
+    const schema::SectionObject& s = h.sections[i];
+    out += std::string(i ? ", " : "") + "{\"begin_offset\": " + std::to_string(s.begin_offset) +
+           ", \"end_offset\": " + std::to_string(s.end_offset) + ", \"data_type\": " + std::to_string(s.data_type) +
+           ", \"data_type_name\": " + JsonString(schema::AnySectionDataTypeToString(s.data_type)) +
+           ", \"items\": " + JsonItems(s.items) + "}";
+  }
+  return out + "]}";
+}
+int GiveBytes(const Status& s, std::string& bytes, uint8_t** data, uint64_t* length, char** err) {
+  if (s.ok()) {
+    *length = bytes.size();
+    *data = static_cast<uint8_t*>(malloc(bytes.size() ? bytes.size() : 1));
+    if (*data) memcpy(*data, bytes.data(), bytes.size());
+  }
+  return Finish(s, err);
+}
+}  // namespace
+
+extern "C" {
+
+// The header of a .litertlm file (path != null) or of a buffer, as JSON text (malloc'd).
+int hle_litertlm_header(const char* path, const void* data, uint64_t length, char** json, char** err) {
+  schema::LitertlmHeader header;
+  Status s = path ? schema::ReadHeaderFromLiteRTLM(std::string(path), &header)
+                  : schema::ReadHeaderFromLiteRTLM(data, static_cast<size_t>(length), &header);
+  if (s.ok()) *json = CopyText(DescribeHeader(header));
+  return Finish(s, err);
+}
+
+// what: 0 section bytes of `expected_type`, 1 HF tokenizer JSON of section idx, 2 the first HF tokenizer JSON,
+// 3 the first generic binary section. *data is malloc'd.
+int hle_litertlm_read(const char* path, int32_t what, int32_t section_idx, int32_t expected_type, uint8_t** data,
+                      uint64_t* length, char** err) {
+  std::string bytes;
+  Status s;
+  switch (what) {
+    case 0: s = schema::ReadSectionBytes(path, section_idx, static_cast<uint8_t>(expected_type), &bytes); break;
+    case 1: s = schema::ReadHfTokenizerJsonFromSection(path, section_idx, &bytes); break;
+    case 2: s = schema::ReadAnyHfTokenizerJson(path, &bytes); break;
+    case 3: s = schema::ReadAnyBinaryData(path, &bytes); break;
+    default: s = InvalidArgumentError("unknown read");
+  }
+  return GiveBytes(s, bytes, data, length, err);
 }
 
 }  // extern "C"
