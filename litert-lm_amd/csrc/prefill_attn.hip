@@ -457,25 +457,41 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // ---- normalise and store: lane (n, hh) holds channels 32*dp + 8*a + 4*hh + b
-  auto store = [&](const f16v (&acc)[NDP], float l_run, int row) {
-    const float l_tot = wave_xor_add(l_run, 32);
+  // ---- normalise and store. Lane (n, hh) holds channels 32*dp + 8*a + 4*hh + b of
+  // query n: written from there, one store instruction would touch 32 rows with
+  // 16 bytes each. The rows go through LDS instead (the rings are idle now; every
+  // wave has its own patch, rows padded to 528 bytes against bank conflicts) and
+  // leave as whole 512-byte rows, two per store instruction.
+  __syncthreads();  // every wave is done with the last V block
+  {
+    constexpr int kRowStride = 2 * D + 16;
+    uint8_t* const patch = smem + wave * (kStretch * kRowStride);
+    const float l_tot = wave_xor_add(l_run0, 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (row < a.n) {
-      elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
 #pragma unroll
-      for (int dp = 0; dp < NDP; ++dp) {
+    for (int dp = 0; dp < NDP; ++dp) {
 #pragma unroll
-        for (int aa = 0; aa < 4; ++aa) {
-          elem_t o[4];
+      for (int aa = 0; aa < 4; ++aa) {
+        elem_t o[4];
 #pragma unroll
-          for (int b = 0; b < 4; ++b) o[b] = (elem_t)(acc[dp][4 * aa + b] * inv);
-          *reinterpret_cast<u2*>(orow + 32 * dp + 8 * aa + 4 * hh) = *reinterpret_cast<const u2*>(o);
-        }
+        for (int b = 0; b < 4; ++b) o[b] = (elem_t)(acc0[dp][4 * aa + b] * inv);
+        *reinterpret_cast<u2*>(patch + n * kRowStride + (32 * dp + 8 * aa + 4 * hh) * 2) = *reinterpret_cast<const u2*>(o);
       }
     }
-  };
-  store(acc0, l_run0, row0);
+    // (the patch is private to the wave and LDS operations of a wave stay in order: no barrier)
+    const int row_base = my_pos0 - a.q_pos0;
+    const int chunk = lane & 31;
+#pragma unroll
+    for (int j = 0; j < kStretch / 2; ++j) {
+      const int r = 2 * j + hh;
+      const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStride + chunk * 16);
+      const int row = row_base + r;
+      if (row < a.n) {
+        elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
+        *reinterpret_cast<u4*>(orow + chunk * 8) = w;
+      }
+    }
+  }
   }  // next work item
 
   // The last workgroup to get here (all others have drawn their final, failed
