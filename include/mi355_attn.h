@@ -236,6 +236,8 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      from the number of workgroups of the launch
  *   "rowwise_prefill"  0/1 run prefill row by row through the decode kernel
  *                      (the only path for fp32 and int8 caches)
+ *   "prefill_workgroups" upper bound of the persistent workgroups of the prefill
+ *                      kernel, 0 (default) = one per compute unit
  */
 int mi355_attn_set_option(mi355_attn* handle, const char* name, int32_t value);
 

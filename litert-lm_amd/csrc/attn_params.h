@@ -130,6 +130,7 @@ struct PrefillArgs {
   int32_t layer_begin, n_layers;
   int32_t seq, q_pos0, n;
   float scale, softcap;
+  int32_t max_workgroups;  // 0 = one per CU; else an upper bound (tests: many work items per workgroup)
 };
 constexpr int kPrefillQueues = 8;                     // one per XCD
 constexpr int kPrefillSchedInts = kPrefillQueues + 1;  // + count of workgroups that are done

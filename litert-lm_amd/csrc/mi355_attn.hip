@@ -104,6 +104,7 @@ struct mi355_attn {
   bool timed = false;
   DecodeTuning tuning;
   bool rowwise_prefill = false;  // force the row-wise prefill path (cross-checks)
+  int prefill_workgroups = 0;    // 0 = one per CU
 };
 
 namespace {
@@ -319,6 +320,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.n = n;
     a.scale = h->cfg.scale;
     a.softcap = h->cfg.softcap;
+    a.max_workgroups = h->prefill_workgroups;
     HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
   } else {
     // Row-wise path (fp32 and int8 caches): every query row is one decode item
@@ -735,6 +737,9 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
     h->tuning.waves = value;
   } else if (!strcmp(name, "rowwise_prefill")) {
     h->rowwise_prefill = value != 0;
+  } else if (!strcmp(name, "prefill_workgroups")) {
+    if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
+    h->prefill_workgroups = value;
   } else {
     return MI355_ATTN_INVALID_ARGUMENT;
   }

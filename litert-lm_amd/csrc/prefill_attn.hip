@@ -64,11 +64,15 @@ struct El<kBF16> {
 // Key (0..31, within a block) that MFMA row m of S^T stands for.
 __device__ __forceinline__ int key_of_row(int m) { return 16 * ((m >> 3) & 1) + 8 * (m >> 4) + (m & 7); }
 
-// LDS plan (dynamic): a ring of three K blocks and a ring of three V blocks,
-// 2 * 3 * 64*D bytes = 96 KiB at head_dim 256.
+// LDS plan (dynamic): a ring of three K blocks and a ring of three V blocks
+// (2 * 3 * 64*D bytes = 96 KiB at head_dim 256), then the query rows of the
+// four waves (64 KiB): 160 KiB, all a CU has.
 constexpr int kStages = 3;
+constexpr int kWaves = 4;       // per workgroup
+constexpr int kStretch = 32;    // query positions per wave: one tile
+
 template <int D>
-constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D; }
+constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D + kWaves * kStretch * 2 * D; }  // rings + query rows
 
 // s_waitcnt immediates (gfx9 encoding: vmcnt[3:0], expcnt[6:4], lgkmcnt[11:8],
 // vmcnt[15:14]) that wait on vector-memory operations only.
@@ -76,8 +80,6 @@ constexpr int kWaitVm0 = 0x0F70;  // all of this wave's transfers have landed
 constexpr int kWaitVm4 = 0x0F74;  // all but the 4 most recent ones
 constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
 
-constexpr int kWaves = 4;       // per workgroup
-constexpr int kStretch = 32;    // query positions per wave: one tile
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.
 template <int... Is, class F>
@@ -107,6 +109,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   // The ticket of the next work item is passed through the last V stage, which
   // no transfer writes before the second barrier of an item.
   volatile int* const sm_ticket = reinterpret_cast<volatile int*>(sm_v + (kStages - 1) * kBlockBytes);
+  uint8_t* const sm_q = smem + 2 * kStages * kBlockBytes;  // [kWaves][kStretch rows of 2 * D bytes]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -165,7 +168,6 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int head = kvh * a.group + hb * HPB + (wave % HPB);
   const int wg_pos0 = a.q_pos0 + tile * (kStretch * PT);  // first position of the workgroup
   const int my_pos0 = wg_pos0 + (wave / HPB) * kStretch;  // first position of this wave's stretch
-  const int row0 = my_pos0 - a.q_pos0 + n;                // query row in q / out
   const int my_pos = my_pos0 + n;
 
   const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
@@ -206,17 +208,22 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   if (nblk > 1) fetch(kplane, sm_k, 1);
   if (nblk > 2) fetch(kplane, sm_k, 2);
 
-  // Q^T operand in registers: slice j of lane (n, hh) holds channels
-  // 16*j + 8*hh .. +7 of the lane's query.
-  vec8 q0[NJ];
+  vec8 q0[NJ];  // Q^T operand, filled from LDS once the rows have landed
+  // The wave's 32 query rows travel to LDS as whole rows, two per transfer
+  // (lanes 0-31 one row, lanes 32-63 the next). Lane l of a transfer asks for the
+  // 16-byte piece (l % 32) ^ (row % 16) of its row, so a row's pieces sit
+  // permuted in LDS and the reads below, 16 lanes on 16 different rows at a
+  // time, fall on 16 different bank groups.
   {
-    const bool ok0 = row0 < a.n;
-    const elem_t* qrow0 =
-        reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + (ok0 ? row0 : 0)) * a.hq + head) * D;
+    uint8_t* const qpatch = sm_q + wave * (kStretch * 2 * D);
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const u4 w0 = *reinterpret_cast<const u4*>(qrow0 + 16 * j + 8 * hh);
-      q0[j] = bit_cast<vec8>(ok0 ? w0 : u4{0, 0, 0, 0});
+    for (int t = 0; t < kStretch / 2; ++t) {
+      const int r = 2 * t + hh;
+      const int row = min(my_pos0 - a.q_pos0 + r, a.n - 1);  // rows past the end repeat the last one; never stored
+      const uint8_t* g = reinterpret_cast<const uint8_t*>(a.q) +
+                         ((((int64_t)li * a.n + row) * a.hq + head) * D) * 2 + ((n ^ (r & 15)) * 16);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                       (__attribute__((address_space(3))) void*)(qpatch + t * 1024), 16, 0, 0);
     }
   }
 
@@ -395,6 +402,14 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();  // the first blocks are resident
 
+  // Q^T operand in registers: slice j of lane (n, hh) holds channels
+  // 16*j + 8*hh .. +7 of the lane's query = piece 2*j + hh of row n.
+  {
+    const uint8_t* const qrow = sm_q + wave * (kStretch * 2 * D) + n * (2 * D);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) q0[j] = *reinterpret_cast<const vec8*>(qrow + (((2 * j + hh) ^ (n & 15)) * 16));
+  }
+
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
   {  // scores of block 0
@@ -538,7 +553,9 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
   }
-  const dim3 grid(items < cus ? items : cus, 1, 1);
+  int wgs = items < cus ? items : cus;
+  if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
+  const dim3 grid(wgs, 1, 1);
   if (hpb == 4) return launch_hpb<DT, D, 4>(a, grid, stream, ev0, ev1);
   if (hpb == 2) return launch_hpb<DT, D, 2>(a, grid, stream, ev0, ev1);
   return launch_hpb<DT, D, 1>(a, grid, stream, ev0, ev1);

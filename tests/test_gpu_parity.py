@@ -322,6 +322,40 @@ def test_prefill_chunked_equals_one_shot_and_layers_call():
         assert orc.rel_err(two.float().cpu().numpy(), one.float().cpu().numpy()) < TOL[A.BF16]
 
 
+@pytest.mark.parametrize("dt", [A.F16, A.BF16])
+@pytest.mark.parametrize("hq,hkv", [(4, 1), (8, 4), (3, 1)])
+def test_prefill_many_work_items_per_workgroup(dt, hq, hkv):
+    """Few persistent workgroups walking many work items each (what one launch over 26 layers does on
+    the full chip): the hand-over between items -- tickets, rings, query rows, output rows -- must not
+    depend on how many workgroups share the queue. Short and long items, ragged ends, local and global
+    layers, a later chunk."""
+    nl, n, pos0 = 5, 333, 160
+    windows = [0, 70, 0, 512, 33]
+    with make(nl, hq, hkv, pos0 + n, 1, dt, layer_window=windows) as at:
+        qd, _ = dev(gen(91, nl, n, hq, D), dt)
+        for layer in range(nl):
+            kd, _ = dev(gen(92 + layer, pos0 + n, hkv, D), dt)
+            vd, _ = dev(gen(97 + layer, pos0 + n, hkv, D), dt)
+            at.kv_append(layer, 0, 0, kd, vd)
+        ref = torch.empty_like(qd)
+        for layer in range(nl):           # one launch per layer, one workgroup per item
+            at.prefill(layer, 0, pos0, n, qd[layer], ref[layer])
+        torch.cuda.synchronize()
+        _, qr = dev(gen(91, nl, n, hq, D), dt)
+        _, kr = dev(gen(92, pos0 + n, hkv, D), dt)
+        _, vr = dev(gen(97, pos0 + n, hkv, D), dt)
+        want = orc.sdpa(qr[0], kr, vr, D ** -0.5, q_pos0=pos0, window=0)
+        assert err_of(ref[0].float().cpu().numpy(), want, dt) < TOL[dt]
+        for wgs in (1, 2, 3, 7):
+            at.set_option("prefill_workgroups", wgs)
+            out = torch.full_like(qd, float("nan"))
+            for _ in range(2):            # twice: the queues reset themselves between launches
+                at.prefill(0, 0, pos0, n, qd, out, n_layers=nl)
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (wgs, hq, hkv)
+        at.set_option("prefill_workgroups", 0)
+
+
 def test_prefill_rowwise_fp32_and_int8():
     L = 200
     with make(1, 4, 1, 256, 1, A.F32, layer_window=[50]) as at:
