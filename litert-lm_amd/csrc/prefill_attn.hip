@@ -81,6 +81,16 @@ constexpr int kWaitVm4 = 0x0F74;  // all but the 4 most recent ones
 constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
 
 
+// Workgroup barrier that orders LDS traffic only. __syncthreads() (and any fence
+// the compiler knows of) also waits for every outstanding vector-memory
+// operation, LDS transfers included: here those are the K / V blocks still on
+// their way into other ring stages, exactly what is meant to stay in flight
+// across a barrier. What must have landed before a barrier is waited for
+// explicitly (s_waitcnt vmcnt) in front of it. The "memory" clobber keeps the
+// compiler from moving memory operations across.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.
 template <int... Is, class F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
@@ -152,7 +162,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     sm_ticket[0] = x;
     sm_ticket[1] = t;
   }
-  __syncthreads();  // also: every wave is done with the LDS rings of the previous item
+  lds_barrier();  // also: every wave is done with the LDS rings of the previous item
   // (uniform values, kept in scalar registers)
   const int qx = __builtin_amdgcn_readfirstlane(sm_ticket[0]);
   const int ticket = __builtin_amdgcn_readfirstlane(sm_ticket[1]);
@@ -400,7 +410,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   };
 
   __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();  // the first blocks are resident
+  lds_barrier();  // the first blocks are resident
 
   // Q^T operand in registers: slice j of lane (n, hh) holds channels
   // 16*j + 8*hh .. +7 of the lane's query = piece 2*j + hh of row n.
@@ -425,6 +435,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     });
     __builtin_amdgcn_sched_barrier(0);
   }
+  lds_barrier();  // every wave has read K block 0: iteration 0 sends a new block into its stage
   auto iteration = [&](int i, auto has_prev, auto has_next) {
     const bool fetch_k = i + 3 < nblk, fetch_v = i + 1 < nblk;
     // The accumulators stay in the AGPR half of the register file; scores,
@@ -443,7 +454,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     if (fetch_k && fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm8);
     else if (fetch_k || fetch_v) __builtin_amdgcn_s_waitcnt(kWaitVm4);
     else __builtin_amdgcn_s_waitcnt(kWaitVm0);
-    __syncthreads();
+    lds_barrier();
   };
   if (nblk == 1) {
     iteration(0, no, no);
@@ -477,7 +488,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   // 16 bytes each. The rows go through LDS instead (the rings are idle now; every
   // wave has its own patch, rows padded to 528 bytes against bank conflicts) and
   // leave as whole 512-byte rows, two per store instruction.
-  __syncthreads();  // every wave is done with the last V block
+  lds_barrier();  // every wave is done with the last V block
   {
     constexpr int kRowStride = 2 * D + 16;
     uint8_t* const patch = smem + wave * (kStretch * kRowStride);
