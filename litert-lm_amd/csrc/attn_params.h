@@ -131,8 +131,14 @@ struct PrefillArgs {
   int32_t seq, q_pos0, n;
   float scale, softcap;
   int32_t max_workgroups;  // 0 = one per CU; else an upper bound (tests: many work items per workgroup)
+  // Units (layer, KV head, head block) in the order the queues deal them out: longest key loops first
+  // (global layers before windowed ones). use_order == 0: identity (more units than the table holds).
+  const int32_t* host_window;  // host copy of layer_window (for the ordering), may be null
+  int32_t use_order;
+  uint16_t unit_order[128];
 };
-constexpr int kPrefillQueues = 8;                     // one per XCD
+constexpr int kPrefillQueues = 2;                     // ticket queues; workgroup k draws from queue k % 2 first
+constexpr int kPrefillOrderUnits = 128;               // entries of PrefillArgs::unit_order
 constexpr int kPrefillSchedInts = kPrefillQueues + 1;  // + count of workgroups that are done
 
 struct KvCopyArgs {

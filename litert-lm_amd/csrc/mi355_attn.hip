@@ -321,6 +321,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.scale = h->cfg.scale;
     a.softcap = h->cfg.softcap;
     a.max_workgroups = h->prefill_workgroups;
+    a.host_window = h->window.data();
     HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
   } else {
     // Row-wise path (fp32 and int8 caches): every query row is one decode item

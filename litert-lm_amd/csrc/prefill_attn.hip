@@ -33,6 +33,9 @@
 #include <type_traits>
 #include <utility>
 
+#include <algorithm>
+#include <vector>
+
 #include "attn_params.h"
 #include "kernels.h"
 #include <hip/hip_ext.h>
@@ -126,11 +129,14 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int n = lane & 31, hh = lane >> 5;
   // Persistent workgroups, one per CU, draw work items = (unit, stretch) from
   // queues of atomic tickets. A unit = (layer, KV head, head block) shares one
-  // K/V plane. Workgroup k runs on XCD k % 8 (round-robin dispatch) and each XCD
-  // has its own L2, so there is one queue per XCD holding every eighth unit, all
-  // stretches of those units, longest key loops first: the K/V blocks a CU asks
-  // for are then mostly in its XCD's L2 already. A workgroup whose own queue has
-  // run dry takes from the others', which evens out the tail.
+  // K/V plane. The units are dealt to the queues in order of decreasing work
+  // (the host sorts them: global layers before windowed ones), and a queue hands
+  // out all stretches of its units, longest key loops first. Workgroup k starts
+  // on queue k % 2, i.e. the workgroups of every other XCD share a queue and the
+  // K/V blocks they ask for are mostly in their XCDs' L2 caches already; a
+  // workgroup whose queue has run dry takes from the other one, which evens out
+  // the tail. (Eight queues, one per XCD, kept the blocks closer but left the
+  // tail 11 % long: with 26 layers a queue held three or four units.)
   const int hblocks = a.group / HPB;
   const int per_layer = a.geom.hkv * hblocks;
   const int units = a.n_layers * per_layer;
@@ -169,7 +175,8 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   if (ticket < 0) break;  // every queue is empty: the only exit, reached by all workgroups
   const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
   const int ti = ticket / qcnt, ui = ticket - ti * qcnt;  // stretch-major: a queue's longest loops first
-  const int u = qx + kPrefillQueues * ui;
+  const int slot = qx + kPrefillQueues * ui;
+  const int u = a.use_order ? a.unit_order[slot] : slot;
   const int li = u / per_layer, rem = u - li * per_layer;
   const int kvh = rem / hblocks, hb = rem - kvh * hblocks;
   const int tile = tiles - 1 - ti;
@@ -564,12 +571,37 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
   }
+  PrefillArgs b = a;
+  b.use_order = 0;
+  const int units = a.n_layers * a.geom.hkv * (G / hpb);
+  if (units <= kPrefillOrderUnits && a.host_window) {
+    // work of a unit = key blocks over all stretches of its layer; stable sort, heaviest first
+    const int per_layer = a.geom.hkv * (G / hpb);
+    const int tiles = (a.n + kStretch * pt - 1) / (kStretch * pt);
+    std::vector<long> work(a.n_layers);
+    for (int li = 0; li < a.n_layers; ++li) {
+      const int w = a.host_window[a.layer_begin + li];
+      long sum = 0;
+      for (int t = 0; t < tiles; ++t) {
+        const int p0 = a.q_pos0 + t * kStretch * pt;
+        const int last = std::min(p0 + kStretch * pt, a.q_pos0 + a.n) - 1;
+        const int lo = (w > 0 && p0 - w + 1 > 0) ? (p0 - w + 1) / kKeysPerBlock : 0;
+        sum += last / kKeysPerBlock - lo + 1;
+      }
+      work[li] = sum;
+    }
+    std::vector<int> order(units);
+    for (int u = 0; u < units; ++u) order[u] = u;
+    std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return work[x / per_layer] > work[y / per_layer]; });
+    for (int u = 0; u < units; ++u) b.unit_order[u] = (uint16_t)order[u];
+    b.use_order = 1;
+  }
   int wgs = items < cus ? items : cus;
   if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
   const dim3 grid(wgs, 1, 1);
-  if (hpb == 4) return launch_hpb<DT, D, 4>(a, grid, stream, ev0, ev1);
-  if (hpb == 2) return launch_hpb<DT, D, 2>(a, grid, stream, ev0, ev1);
-  return launch_hpb<DT, D, 1>(a, grid, stream, ev0, ev1);
+  if (hpb == 4) return launch_hpb<DT, D, 4>(b, grid, stream, ev0, ev1);
+  if (hpb == 2) return launch_hpb<DT, D, 2>(b, grid, stream, ev0, ev1);
+  return launch_hpb<DT, D, 1>(b, grid, stream, ev0, ev1);
 }
 
 }  // namespace
