@@ -333,6 +333,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="headline decode workload only")
+    ap.add_argument("--no-pipeline", action="store_true",
+                    help="skip the 1024 / 256 protocol run through the C++ executor (thousands of small launches: "
+                         "left out of rocprofv3 runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for rocprofv3 --pmc counters)")
     args = ap.parse_args()
@@ -438,15 +441,16 @@ def main():
         log(f"[bench] {pa['workload']}: {pa['ms_per_step']*1e3:.1f} us/step, kernel {pa['kernel_ms']*1e3:.1f} us "
             f"({pa['kernel_GBps']:.0f} GB/s), one token {pa['single_token_latency_us']:.1f} us")
         result["pre_attention"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in pa.items()}
-        text, pre_tps, dec_tps = pipeline_report(load_package().executor)
-        log("[bench] the reference's benchmark protocol (1024 prefill / 256 decode ids) through the C++ executor,\n"
-            "        synthetic host-side layers around the HIP attention path, host tensors staged per call:\n" + text)
-        result["pipeline_protocol"] = {
-            "what": "1024 prefill ids + 256 decode steps through HipLlmExecutor (26 layers, 5 local : 1 global, fp16, "
-                    "fused step before attention); layers other than attention are host-side synthetic stand-ins and "
-                    "every call stages host tensors: an end-to-end protocol run in the reference's report format, "
-                    "not a kernel figure",
-            "prefill_tokens_per_s": pre_tps, "decode_tokens_per_s": dec_tps}
+        if not args.no_pipeline:
+            text, pre_tps, dec_tps = pipeline_report(load_package().executor)
+            log("[bench] the reference's benchmark protocol (1024 prefill / 256 decode ids) through the C++ executor,\n"
+                "        synthetic host-side layers around the HIP attention path, host tensors staged per call:\n" + text)
+            result["pipeline_protocol"] = {
+                "what": "1024 prefill ids + 256 decode steps through HipLlmExecutor (26 layers, 5 local : 1 global, fp16, "
+                        "fused step before attention); layers other than attention are host-side synthetic stand-ins and "
+                        "every call stages host tensors: an end-to-end protocol run in the reference's report format, "
+                        "not a kernel figure",
+                "prefill_tokens_per_s": pre_tps, "decode_tokens_per_s": dec_tps}
 
     if not args.no_cpu:
         cpu = cpu_baseline_c3(dec["layers"], 4096, dec["step_bytes"])
