@@ -356,6 +356,30 @@ def test_prefill_many_work_items_per_workgroup(dt, hq, hkv):
         at.set_option("prefill_workgroups", 0)
 
 
+def test_prefill_more_units_than_the_order_table_holds():
+    """40 layers x 4 KV heads = 160 units: the launch falls back to the identity order of the units
+    (the host-sorted order table holds 128); every layer still has to come out right."""
+    nl, n, hq, hkv, dt = 40, 70, 8, 4, A.F16
+    windows = [0 if l % 3 == 0 else 20 + l for l in range(nl)]
+    with make(nl, hq, hkv, n, 1, dt, layer_window=windows) as at:
+        qd, qr = dev(gen(111, nl, n, hq, D), dt)
+        kd, kr = dev(gen(112, n, hkv, D), dt)
+        vd, vr = dev(gen(113, n, hkv, D), dt)
+        for layer in range(nl):
+            at.kv_append(layer, 0, 0, kd, vd)
+        out = torch.empty_like(qd)
+        at.prefill(0, 0, 0, n, qd, out, n_layers=nl)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        for layer in (0, 1, 17, 38, 39):
+            want = orc.sdpa(qr[layer], kr, vr, D ** -0.5, window=windows[layer])
+            assert err_of(got[layer], want, dt) < TOL[dt], layer
+        per = torch.empty_like(qd[5])
+        at.prefill(5, 0, 0, n, qd[5], per)
+        torch.cuda.synchronize()
+        assert torch.equal(per, out[5])
+
+
 def test_prefill_rowwise_fp32_and_int8():
     L = 200
     with make(1, 4, 1, 256, 1, A.F32, layer_window=[50]) as at:
