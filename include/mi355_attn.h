@@ -238,6 +238,11 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      (the only path for fp32 and int8 caches)
  *   "prefill_workgroups" upper bound of the persistent workgroups of the prefill
  *                      kernel, 0 (default) = one per compute unit
+ *   "prefill_bf16_single_p" 0 (default): a bf16 prefill feeds each probability to
+ *                      the P.V product as a high and a low bf16 part, which keeps the
+ *                      result within the output format's own rounding; 1: one bf16
+ *                      operand per probability (a third fewer MFMAs; adds ~1.5e-3
+ *                      L2-relative error, the usual trade of bf16 attention kernels)
  */
 int mi355_attn_set_option(mi355_attn* handle, const char* name, int32_t value);
 

@@ -135,6 +135,7 @@ struct PrefillArgs {
   // (global layers before windowed ones). use_order == 0: identity (more units than the table holds).
   const int32_t* host_window;  // host copy of layer_window (for the ordering), may be null
   int32_t use_order;
+  int32_t single_p;  // bf16: probabilities enter P.V as one bf16 operand (faster, ~1.5e-3 L2 error) instead of two
   uint16_t unit_order[128];
 };
 constexpr int kPrefillQueues = 2;                     // ticket queues; workgroup k draws from queue k % 2 first

@@ -105,6 +105,7 @@ struct mi355_attn {
   DecodeTuning tuning;
   bool rowwise_prefill = false;  // force the row-wise prefill path (cross-checks)
   int prefill_workgroups = 0;    // 0 = one per CU
+  bool bf16_single_p = false;    // bf16 prefill: one MFMA operand per probability instead of a high and a low part
 };
 
 namespace {
@@ -321,6 +322,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.scale = h->cfg.scale;
     a.softcap = h->cfg.softcap;
     a.max_workgroups = h->prefill_workgroups;
+    a.single_p = h->bf16_single_p ? 1 : 0;
     a.host_window = h->window.data();
     HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
   } else {
@@ -741,6 +743,8 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   } else if (!strcmp(name, "prefill_workgroups")) {
     if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_workgroups = value;
+  } else if (!strcmp(name, "prefill_bf16_single_p")) {
+    h->bf16_single_p = value != 0;
   } else {
     return MI355_ATTN_INVALID_ARGUMENT;
   }

@@ -104,7 +104,7 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-template <int DT, int D, int HPB, bool CAP>
+template <int DT, int D, int HPB, bool CAP, bool SPLITP>
 __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
@@ -114,7 +114,8 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   constexpr int NDP = D / 32;            // 32-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;    // one 32-key block of a 16-bit plane
   constexpr int kXfers = 16 / kWaves;    // 1 KiB transfers per wave, block and plane
-  constexpr int NP = DT == kBF16 ? 4 : 2;  // P operands per tile: p0, p1 (+ low parts for bf16)
+  // P operands per tile: p0, p1, and with SPLITP (bf16 only) their low parts
+  constexpr int NP = SPLITP ? 4 : 2;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint8_t* const sm_k = smem;                              // [kStages][K block]
@@ -342,15 +343,18 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
       } else {
         constexpr int e = P - 18;
         sa[e] = fast_exp2(fmaf(sa[e], c, neg_m));
+        // one bf16 operand per probability: the row sum is taken over the rounded
+        // values, so that the rounding cancels where a few keys carry the row
+        if constexpr (DT == kBF16 && !SPLITP) sa[e] = (float)(elem_t)sa[e];
         lsum += sa[e];
         if constexpr (e & 1) {
-          // probabilities as MFMA operands (bf16: high and low parts, 8
-          // significant bits alone would put ~1e-3 of relative error into P.V)
+          // probabilities as MFMA operands (bf16 with SPLITP: high and low parts, 8
+          // significant bits alone put ~1.5e-3 of relative error into P.V)
 #pragma unroll
           for (int ee = e - 1; ee <= e; ++ee) {
             const elem_t hi = (elem_t)sa[ee];
             p_cur[ee >> 3][ee & 7] = hi;
-            if constexpr (DT == kBF16) p_cur[2 + (ee >> 3)][ee & 7] = (elem_t)(sa[ee] - (float)hi);
+            if constexpr (NP == 4) p_cur[2 + (ee >> 3)][ee & 7] = (elem_t)(sa[ee] - (float)hi);
           }
         }
         // Pins: without them the compiler sinks this arithmetic, whose results
@@ -358,7 +362,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
         asm volatile("" : "+v"(sa[e]), "+v"(lsum));
         if constexpr ((e & 7) == 7) {
           asm volatile("" : "+v"(p_cur[e >> 3]));
-          if constexpr (DT == kBF16) asm volatile("" : "+v"(p_cur[2 + (e >> 3)]));
+          if constexpr (NP == 4) asm volatile("" : "+v"(p_cur[2 + (e >> 3)]));
         }
       }
     };
@@ -536,26 +540,31 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   }
 }
 
-template <int DT, int D, int HPB, bool CAP>
+template <int DT, int D, int HPB, bool CAP, bool SPLITP>
 hipError_t launch_variant(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill_lds_bytes<D>();
   static bool configured = false;  // more than 64 KiB of LDS has to be requested once per kernel
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB, CAP>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB, CAP, SPLITP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
     configured = true;
   }
   // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
-  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB, CAP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
+  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB, CAP, SPLITP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
                         a);
   return hipGetLastError();
 }
 
 template <int DT, int D, int HPB>
 hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
-  return a.softcap > 0.f ? launch_variant<DT, D, HPB, true>(a, grid, stream, ev0, ev1)
-                         : launch_variant<DT, D, HPB, false>(a, grid, stream, ev0, ev1);
+  if constexpr (DT == kBF16) {
+    if (!a.single_p)
+      return a.softcap > 0.f ? launch_variant<DT, D, HPB, true, true>(a, grid, stream, ev0, ev1)
+                             : launch_variant<DT, D, HPB, false, true>(a, grid, stream, ev0, ev1);
+  }
+  return a.softcap > 0.f ? launch_variant<DT, D, HPB, true, false>(a, grid, stream, ev0, ev1)
+                         : launch_variant<DT, D, HPB, false, false>(a, grid, stream, ev0, ev1);
 }
 
 template <int DT, int D>

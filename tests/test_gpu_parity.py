@@ -287,6 +287,34 @@ def test_prefill_small_shapes(dt, hq, hkv):
         say(f"prefill small dt={dt} hq={hq} hkv={hkv}: ok")
 
 
+def test_prefill_bf16_one_operand_per_probability():
+    # option "prefill_bf16_single_p": P enters the P.V product as one bf16 value. Error beyond the output
+    # format's own rounding stays under 2e-3 (max-norm); with the output rounding the L2 figure is
+    # 2.0e-3 .. 2.5e-3 (the default, split, path stays under 2e-3, see err_of), bound here at 3e-3.
+    # A row that sees one key returns that key's V bit-exactly: the row sum is taken over the rounded values.
+    L, hq, hkv = 1024, 4, 1
+    windows = [0, 512, 1]
+    with make(len(windows), hq, hkv, L, 1, A.BF16, layer_window=windows) as at:
+        at.set_option("prefill_bf16_single_p", 1)
+        k, v = gen(161, L, hkv, D), gen(162, L, hkv, D)
+        for layer, w in enumerate(windows):
+            kr, vr = fill_seq(at, A.BF16, layer, 0, k, v)
+            for q_pos0, n in ((0, 1024), (129, 200), (1023, 1)):
+                qd, qr = dev(gen(2000 + n, n, hq, D), A.BF16)
+                out = torch.empty_like(qd)
+                at.prefill(layer, 0, q_pos0, n, qd, out)
+                torch.cuda.synchronize()
+                got = out.float().cpu().numpy()
+                ref = c_oracle.sdpa_f64(qr, kr, vr, D ** -0.5, q_pos0=q_pos0, window=w, kv_len=q_pos0 + n)
+                if w == 1:
+                    want = np.broadcast_to(vr[q_pos0:q_pos0 + n, 0][:, None, :], got.shape)
+                    assert np.array_equal(got, want)
+                    continue
+                beyond, l2 = orc.rel_err_beyond_bf16_rounding(got, ref), orc.l2_rel_err(got, ref)
+                say(f"single-P bf16 window={w} q_pos0={q_pos0} n={n}: beyond-rounding {beyond:.3e}, L2 {l2:.3e}")
+                assert beyond < TOL[A.BF16] and l2 < 3e-3
+
+
 def test_prefill_c2_full_size_local_and_global():
     # config 2: 1024-token chunk, Hq4/Hkv1, bf16; one local (W=512) and one global layer
     seed = orc.SEED_BASE + 1
