@@ -15,13 +15,14 @@
 // wave reports the ceil(k/16)-th largest of its 64 maxima (DPP reductions); at
 // least k logits of the segment reach the smallest of those 16 numbers, so only
 // what reaches it - a few hundred candidates - is packed as (order-preserving
-// key, index) words, ranked by counting in LDS (no sort), and the segment's k
-// best go to a workspace. Segments for which that bound is too weak (more than
-// 2048 candidates: long runs of equal values) or that hold fewer than k numbers
-// fall back to a radix descent on the keys with LDS histograms (12 + 12 + 8
-// bits); exact ties at the k-th value are then taken in ascending index order.
-// finish_kernel: one workgroup per row merges the segments' candidates the same
-// way and walks the k winners in the reference's op order.
+// key, index) words. Up to 256 of them go to a workspace as they are; more are
+// ranked by counting in LDS (no sort) and the segment's k best go there.
+// Segments for which that bound is too weak (more than 2048 candidates: long
+// runs of equal values) or that hold fewer than k numbers fall back to a radix
+// descent on the keys with LDS histograms (12 + 12 + 8 bits); exact ties at the
+// k-th value are then taken in ascending index order.
+// finish_kernel: one workgroup per row thresholds and ranks the segments'
+// candidates the same way and walks the k winners in the reference's op order.
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <float.h>
@@ -45,7 +46,8 @@ constexpr int kBins = 4096;
 constexpr int kCap = 2048;              // candidates of one segment that fit in LDS for the sort
 constexpr int kMaxK = MI355_SAMPLER_MAX_K;
 constexpr int kMaxSegments = 16;
-constexpr int kMergeCap = kMaxSegments * kMaxK;  // 4096 candidates of one row in finish_kernel
+constexpr int kSlots = kMaxK;            // workspace words per segment; a zero word is an empty slot
+constexpr int kMergeCap = kMaxSegments * kSlots;  // 4096 words of one row in finish_kernel
 constexpr int kResident = 16;           // logits per thread that stay in registers between the passes
 constexpr int kSegmentMin = kThreads * kResident;  // a segment is this long unless the row needs more than kMaxSegments
 
@@ -58,7 +60,7 @@ struct SamplerArgs {
   float* scores;          // [batch] or null
   int32_t* topk_idx;      // [batch][k] or null
   float* topk_prob;       // [batch][k] or null
-  u64* workspace;         // [batch][segments][k] candidates, (key << 32) | ~index
+  u64* workspace;         // [batch][segments][kSlots] candidates, (key << 32) | ~index, 0 = empty
   int32_t vocab, k, segments, seg_len;
   float p, temperature;
   uint32_t seed;
@@ -181,22 +183,49 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 }
 
 // A lower bound that at least k of the values v (one per thread, 0 = none) reach:
-// every wave reports the j-th largest of its 64 values, j = ceil(k / 16); at
-// least 16 j >= k values reach the smallest of those 16 numbers. One barrier.
-__device__ __forceinline__ uint32_t lower_bound_of_kth(uint32_t v, int k, uint32_t* wave_val, int tid) {
+// each of the first `waves` waves reports the j-th largest of its 64 values,
+// j = ceil(k / waves); at least waves * j >= k values reach the smallest of those
+// numbers (0, a bound that everything reaches, if a wave holds fewer than j
+// values). The values of the other waves are not looked at. One barrier.
+__device__ __forceinline__ uint32_t lower_bound_of_kth(uint32_t v, int k, int waves, uint32_t* wave_val, int tid) {
   const int lane = tid & 63, wave = tid >> 6;
-  const int j_th = (k + kWavesPerWg - 1) / kWavesPerWg;
-  uint32_t m = 0;
-  for (int r = 0; r < j_th; ++r) {
-    m = wave_max_u32(v);
-    const u64 holders = __ballot(v == m);
-    if (lane == __ffsll((long long)holders) - 1) v = 0;  // drop one holder of the maximum
+  const int j_th = (k + waves - 1) / waves;
+  if (j_th > 16) {  // few waves: at most 64 * waves values anyway, and the rounds below cost more than they save
+    __syncthreads();
+    return 0;
   }
-  if (lane == 0) wave_val[wave] = m;
+  if (wave < waves) {
+    uint32_t m = 0;
+    for (int r = 0; r < j_th && (r == 0 || m != 0); ++r) {
+      m = wave_max_u32(v);
+      const u64 holders = __ballot(v == m);
+      if (lane == __ffsll((long long)holders) - 1) v = 0;  // drop one holder of the maximum
+    }
+    if (lane == 0) wave_val[wave] = m;
+  }
   __syncthreads();
   uint32_t tau = wave_val[0];
-  for (int w = 1; w < kWavesPerWg; ++w) tau = min(tau, wave_val[w]);
+  for (int w = 1; w < waves; ++w) tau = min(tau, wave_val[w]);
   return tau;
+}
+
+// Number of set bits of `mask` below this lane.
+__device__ __forceinline__ uint32_t lanes_below(u64 mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+// List slots for the values of a wave that pass a test: take[e] = ballot of value e
+// passing. One atomic per wave on the list's length (an atomic per thread on one
+// address is compiled to a loop over the lanes); returns the wave's first slot, value
+// e of a passing lane goes to first + (set bits of take[0..e)) + lanes_below(take[e]).
+template <int NV>
+__device__ __forceinline__ uint32_t reserve_slots(const u64 (&take)[NV], uint32_t* length, int lane) {
+  uint32_t total = 0;
+#pragma unroll
+  for (int e = 0; e < NV; ++e) total += (uint32_t)__popcll(take[e]);
+  uint32_t first = 0;
+  if (lane == 0 && total) first = atomicAdd(length, total);
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
 }
 
 // The float version (-inf = none): used on the logits themselves.
@@ -216,28 +245,35 @@ __device__ __forceinline__ float lower_bound_of_kth_f32(float v, int k, float* w
   return tau;
 }
 
+constexpr int kRankParts = 8;            // threads that share the comparisons of one candidate, at most
+constexpr int kRankPad = 8 * kRankParts;  // zero words a candidate list needs behind its last entry
+
 // top[r] = the candidate of rank r (number of larger candidates; the words are
-// distinct) for r < k, by counting instead of sorting: 256 candidates at a
-// time, the comparisons of each split over 4 threads.
+// distinct and not zero) for r < k, by counting instead of sorting. Up to 1024
+// candidates at a time, the comparisons of each split over min(8, 1024 / n)
+// threads in runs of a multiple of 8 words. cand[n .. n + kRankPad) are zero
+// words (a zero is larger than nothing, so the runs need no bounds), cand is
+// 16-byte aligned, and rank_sm[] is all zero on entry (both written before the
+// caller's last barrier). Ends with a barrier.
 __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, int k, uint32_t* rank_sm, int tid) {
-  // `width` candidates at a time (a power of two, 128 .. 1024), the comparisons of each split over 1024 / width threads
-  int width = 128;
-  while (width < n && width < kThreads) width <<= 1;
-  const int parts = kThreads / width;
-  const int slot = tid & (width - 1), part = tid / width;
-  const int span = (n + parts - 1) / parts, j0 = part * span, j1 = min(n, j0 + span);
+  const int width = max(1, min(n, kThreads));
+  const int parts = min(kRankParts, kThreads / width);
+  const int slot = tid % width, part = tid / width;
+  const int span = ((n + parts - 1) / parts + 7) & ~7, j0 = part * span;
   for (int blk = 0; blk < n; blk += width) {
-    if (tid < width) rank_sm[tid] = 0;
-    __syncthreads();
-    if (blk + slot < n) {
+    if (blk > 0) {
+      if (tid < width) rank_sm[tid] = 0;
+      __syncthreads();
+    }
+    if (part < parts && blk + slot < n) {
       const u64 c = cand[blk + slot];
       uint32_t cnt = 0;
-      for (int j = j0; j < j1; j += 8) {  // eight independent LDS reads in flight
-        u64 x[8];
+      for (int j = j0; j < j0 + span; j += 8) {  // (the same words for every lane of a wave: broadcast reads)
+        ulonglong2 x[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = j + u < j1 ? cand[j + u] : 0;
+        for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const ulonglong2*>(cand + j + 2 * u);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) cnt += x[u] > c ? 1u : 0u;
+        for (int u = 0; u < 4; ++u) cnt += (x[u].x > c ? 1u : 0u) + (x[u].y > c ? 1u : 0u);
       }
       if (cnt) atomicAdd(&rank_sm[slot], cnt);
     }
@@ -247,7 +283,9 @@ __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, in
   }
 }
 
-// The k largest logits of one segment of one row, sorted, into the workspace.
+// The candidates of one segment of one row into the workspace: everything that
+// reaches the threshold when that is at most kSlots words (the usual case: the
+// row's kernel ranks them anyway), else the segment's k largest.
 // RESIDENT: every segment has at most kSegmentMin logits (the host knows), which
 // then stay in registers; the other instantiation re-reads them (from L2) per pass.
 // 64 registers at most, so that two workgroups share a compute unit.
@@ -255,7 +293,7 @@ template <bool RESIDENT>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
 select_kernel(const SamplerArgs a) {
   __shared__ uint32_t hist[kBins];
-  __shared__ u64 cand[kCap];
+  __shared__ __align__(16) u64 cand[kCap + kRankPad];  // zero behind the last candidate (rank_select)
   __shared__ u64 top[kMaxK];
   __shared__ uint32_t rank_sm[kThreads];
   __shared__ uint32_t wave_sum[kWavesPerWg];
@@ -269,7 +307,7 @@ select_kernel(const SamplerArgs a) {
   const int k = min(a.k, len);
   const float* seg = a.logits + (size_t)b * a.vocab + index0;
   const bool vec_ok = (a.vocab % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
-  u64* out = a.workspace + ((size_t)b * a.segments + sgm) * a.k;
+  u64* out = a.workspace + ((size_t)b * a.segments + sgm) * kSlots;
 
   // A segment of up to 16 logits per thread is read from memory once and stays in
   // registers for all later passes (same index layout as for_each_key); slots past
@@ -315,11 +353,13 @@ select_kernel(const SamplerArgs a) {
       for (int w = 1; w < kWavesPerWg; ++w) best = max(best, cand[w]);
       out[0] = best;
     }
-    for (int i = 1 + tid; i < a.k; i += kThreads) out[i] = 0;
+    for (int i = 1 + tid; i < kSlots; i += kThreads) out[i] = 0;
     return;
   }
 
   // ---- a threshold from the per-thread maxima, then everything that reaches it
+  rank_sm[tid] = 0;  // (for rank_select, as the zeros behind the candidates; barriers follow on every path)
+  for (int i = tid; i < kCap + kRankPad; i += kThreads) cand[i] = 0;
   if constexpr (resident) {
     // on the logits themselves: three instructions per logit, keys only for the candidates
     float tmax = -INFINITY;
@@ -327,26 +367,27 @@ select_kernel(const SamplerArgs a) {
     for (int e = 0; e < kResident; ++e) tmax = fmaxf(tmax, xreg[e]);
     if (tid == 0) n_cand = 0;
     const float tau = lower_bound_of_kth_f32(tmax, k, reinterpret_cast<float*>(wave_sum), tid);  // (barrier inside)
-    uint32_t mine = 0;
+    u64 take[kResident];
 #pragma unroll
-    for (int e = 0; e < kResident; ++e) mine += xreg[e] >= tau ? 1u : 0u;
-    uint32_t pos = mine ? atomicAdd(&n_cand, mine) : 0u;
-    if (mine) {
+    for (int e = 0; e < kResident; ++e) take[e] = __ballot(xreg[e] >= tau);
+    uint32_t slot0 = reserve_slots(take, &n_cand, lane);
 #pragma unroll
-      for (int u = 0; u < kResident / 4; ++u)
+    for (int u = 0; u < kResident / 4; ++u)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (xreg[4 * u + j] >= tau) {
-            if (pos < (uint32_t)kCap) cand[pos] = pack(key_of(xreg[4 * u + j]), index0 + u * kPerIter + tid * 4 + j);
-            ++pos;
-          }
-    }
+      for (int j = 0; j < 4; ++j) {
+        const int e = 4 * u + j;
+        if (take[e]) {  // (uniform over the wave; most are zero)
+          const uint32_t pos = slot0 + lanes_below(take[e]);
+          if (xreg[e] >= tau && pos < (uint32_t)kCap) cand[pos] = pack(key_of(xreg[e]), index0 + u * kPerIter + tid * 4 + j);
+          slot0 += (uint32_t)__popcll(take[e]);
+        }
+      }
     __syncthreads();
   } else {
     uint32_t tmax = 0;
     each([&](uint32_t key, int) { tmax = max(tmax, key); });
     if (tid == 0) n_cand = 0;
-    const uint32_t tau = lower_bound_of_kth(tmax, k, wave_sum, tid);  // (barrier inside)
+    const uint32_t tau = lower_bound_of_kth(tmax, k, kWavesPerWg, wave_sum, tid);  // (barrier inside)
     uint32_t mine = 0;
     each([&](uint32_t key, int) { mine += key >= tau ? 1u : 0u; });
     uint32_t pos = mine ? atomicAdd(&n_cand, mine) : 0u;
@@ -358,8 +399,13 @@ select_kernel(const SamplerArgs a) {
     });
     __syncthreads();
   }
+  // (n_cand is only written again behind further barriers)
   const bool fast_ok = n_cand <= (uint32_t)kCap && n_cand >= (uint32_t)k;  // (fewer than k: NaNs among the logits)
-  __syncthreads();
+  if (fast_ok && n_cand <= (uint32_t)kSlots) {
+    const int n = (int)n_cand;
+    if (tid < kSlots) out[tid] = tid < n ? cand[tid] : 0;
+    return;
+  }
 
   if (!fast_ok) {
     // ---- radix descent: (mask, val) = the key prefix of the k-th largest value so far
@@ -387,6 +433,7 @@ select_kernel(const SamplerArgs a) {
     // ---- collection: everything above the prefix, and the prefix bin itself
     // (of exact ties only the `need` lowest indices)
     if (tid == 0) { n_cand = 0; n_ties = 0; }
+    for (int i = tid; i < kCap + kRankPad; i += kThreads) cand[i] = 0;
     __syncthreads();
     if (!exact_ties) {
       each([&](uint32_t key, int i) {
@@ -430,44 +477,57 @@ select_kernel(const SamplerArgs a) {
   }
   const int n = (int)n_cand;  // k <= n <= kCap
   rank_select(cand, n, top, k, rank_sm, tid);
-  for (int i = tid; i < a.k; i += kThreads) out[i] = i < k ? top[i] : 0;
+  if (tid < kSlots) out[tid] = tid < k ? top[tid] : 0;
 }
 
 // Merges the segments' candidates of one row and draws (sampling_cpu_util.cc:98-131, 189-230).
 __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
-  __shared__ u64 surv[kMergeCap];  // the segments' candidates that reach the threshold
+  __shared__ __align__(16) u64 surv[kMergeCap + kRankPad];  // the segments' candidates that reach the threshold, then zeros
   __shared__ u64 cand[kMaxK];      // the row's k winners, descending
-  __shared__ float e_sm[kMaxK];
+  __shared__ __align__(16) float e_sm[kMaxK + 16];  // (+16: the loops below read up to 15 entries past the last one they use)
   __shared__ uint32_t rank_sm[kThreads];
   __shared__ uint32_t wave_val[kWavesPerWg];
   __shared__ uint32_t n_surv;
   __shared__ float inv_sm;
   __shared__ double cum_sm[kMaxK];
-  __shared__ int first_reach, first_hit;
-  const int tid = threadIdx.x, b = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, b = blockIdx.x;
   const int k = min(a.k, a.vocab);
-  const int n = a.segments * a.k;  // <= kMergeCap: up to 4 words per thread; zero words are empty slots
+  // Wave s holds the kSlots words of segment s, four consecutive ones per thread;
+  // zero words are empty slots (a segment fills its slots from the front).
+  const int n = a.segments * kSlots;  // <= kMergeCap
   const u64* in = a.workspace + (size_t)b * n;
   u64 w[4];
   uint32_t wmax = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    w[j] = tid + j * kThreads < n ? in[tid + j * kThreads] : 0;
-    wmax = max(wmax, (uint32_t)(w[j] >> 32));
+  if (4 * tid < n) {
+    const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(in + 4 * tid);
+    const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(in + 4 * tid + 2);
+    w[0] = lo.x; w[1] = lo.y; w[2] = hi.x; w[3] = hi.y;
+  } else {
+    w[0] = w[1] = w[2] = w[3] = 0;
   }
-  if (tid == 0) { n_surv = 0; first_reach = k - 1; first_hit = kMaxK; }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) wmax = max(wmax, (uint32_t)(w[j] >> 32));
+  if (tid == 0) n_surv = 0;
+  rank_sm[tid] = 0;  // (for rank_select)
+  for (int i = tid; i < kMergeCap + kRankPad; i += kThreads) surv[i] = 0;
   // same scheme as in select_kernel: a lower bound of the k-th largest key, the
   // words that reach it, their ranks by counting
-  const uint32_t tau = lower_bound_of_kth(wmax, k, wave_val, tid);  // (barrier inside)
-  uint32_t mine = 0;
+  static_assert(kSlots == 4 * 64, "one wave of four-word threads per segment");
+  const uint32_t tau = lower_bound_of_kth(wmax, k, a.segments, wave_val, tid);  // (barrier inside)
+  u64 take[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) mine += (w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau) ? 1u : 0u;
-  uint32_t pos = mine ? atomicAdd(&n_surv, mine) : 0u;
+  for (int j = 0; j < 4; ++j) take[j] = __ballot(w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau);
+  uint32_t slot0 = reserve_slots(take, &n_surv, lane);
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau) surv[pos++] = w[j];
+  for (int j = 0; j < 4; ++j) {
+    if (w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau) surv[slot0 + lanes_below(take[j])] = w[j];
+    slot0 += (uint32_t)__popcll(take[j]);
+  }
   __syncthreads();
   rank_select(surv, (int)n_surv, cand, k, rank_sm, tid);
+  // The rest is the work of k threads: the other waves leave (a barrier waits
+  // only for the waves of the workgroup that are still running).
+  if (tid >= ((k + 63) & ~63)) return;
 
   if (k == 1) {
     if (tid == 0) {
@@ -483,6 +543,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
   const float m = logit_of((uint32_t)(cand[0] >> 32));
   const float t_soft = fmaxf(a.temperature, FLT_EPSILON);
   if (tid < k) e_sm[tid] = expf((logit_of((uint32_t)(cand[tid] >> 32)) - m) / t_soft);
+  if (tid < 16) e_sm[k + tid] = 0.f;
   __syncthreads();
   if (tid == 0) {
     // sequential float32 sum, as the reference; the LDS reads run ahead of the adds
@@ -490,7 +551,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
     for (int i = 0; i < k; i += 8) {
       float x[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) x[u] = i + u < k ? e_sm[i + u] : 0.f;
+      for (int u = 0; u < 8; ++u) x[u] = e_sm[i + u];  // zeros behind entry k - 1
 #pragma unroll
       for (int u = 0; u < 8; ++u) sum += x[u];
     }
@@ -505,29 +566,52 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
   // Cumulative probabilities in float64, every thread summing its own prefix in
   // the reference's order; the nucleus ends at the first one that reaches p, the
   // draw picks the first one that covers it (sampling_cpu_util.cc:189-230).
+  bool reaches = false;
   if (tid < k) {
     double c = 0.0;
-    for (int i = 0; i <= tid; i += 8) {
-      float x[8];
+    for (int i = 0; i <= tid; i += 16) {
+      // 16 probabilities per round trip; conversion and selection are off the chain of additions
+      float4 x[4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) x[u] = i + u <= tid ? e_sm[i + u] : 0.f;
+      for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const float4*>(&e_sm[i + 4 * u]);
+      double d[16];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) c += (double)x[u];
+      for (int u = 0; u < 4; ++u) {
+        d[4 * u] = i + 4 * u <= tid ? (double)x[u].x : 0.0;  // (+0.0 leaves c >= 0 as it is)
+        d[4 * u + 1] = i + 4 * u + 1 <= tid ? (double)x[u].y : 0.0;
+        d[4 * u + 2] = i + 4 * u + 2 <= tid ? (double)x[u].z : 0.0;
+        d[4 * u + 3] = i + 4 * u + 3 <= tid ? (double)x[u].w : 0.0;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) c += d[u];
     }
     cum_sm[tid] = c;
-    if (c >= (double)a.p) atomicMin(&first_reach, tid);
+    reaches = c >= (double)a.p;
+  }
+  // the first thread of all that reaches p (k - 1 if none does: then the nucleus is all k candidates)
+  const int k_waves = (k + 63) >> 6;  // the waves that are still here
+  {
+    const u64 m = __ballot(reaches);
+    if (lane == 0) wave_val[wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
   }
   __syncthreads();
-  const int nucleus = first_reach + 1;  // first_reach starts at k - 1: never reached = all k candidates
+  int first_reach = k - 1;
+  for (int wv = 0; wv < k_waves; ++wv) first_reach = min(first_reach, (int)wave_val[wv]);
+  const int nucleus = first_reach + 1;
   const double mass = cum_sm[first_reach];
   float u01;
   if (a.uniforms) u01 = a.uniforms[b];
   else u01 = (float)(philox_first_word((uint32_t)b, (uint32_t)a.call_index, (uint32_t)(a.call_index >> 32), 0u, a.seed,
                                        0x4D493335u) >> 8) * (1.f / 16777216.f);
   const double draw = (double)u01 * mass;
-  if (tid < nucleus && draw <= cum_sm[tid]) atomicMin(&first_hit, tid);
+  {
+    const u64 m = __ballot(tid < nucleus && draw <= cum_sm[tid]);
+    if (lane == 0) wave_val[8 + wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
+  }
   __syncthreads();
   if (tid == 0) {
+    int first_hit = kMaxK;
+    for (int wv = 0; wv < k_waves; ++wv) first_hit = min(first_hit, (int)wave_val[8 + wv]);
     const int chosen = mass > DBL_EPSILON ? min(first_hit, nucleus - 1) : 0;
     if (a.ids) a.ids[b] = index_of(cand[chosen]);
     if (a.scores) a.scores[b] = logf(expf((logit_of((uint32_t)(cand[chosen] >> 32)) - m) / a.temperature));
@@ -693,10 +777,12 @@ int mi355_sampler_create(const mi355_sampler_config* c, mi355_sampler** out, cha
   if ((e = hipEventCreate(&h->ev0)) != hipSuccess || (e = hipEventCreate(&h->ev1)) != hipSuccess)
     return bail(MI355_SAMPLER_INTERNAL, "hipEventCreate", e);
   // segments of kSegmentMin logits or less (a multiple of 4), unless that would take more than kMaxSegments
-  h->segments = std::max(1, std::min(kMaxSegments, (c->vocab_size + kSegmentMin - 1) / kSegmentMin));
+  // 1, 2, 4, 8 or 16 segments (with three, the row's kernel could not bound its candidates: lower_bound_of_kth)
+  h->segments = 1;
+  while (h->segments < kMaxSegments && (size_t)h->segments * kSegmentMin < (size_t)c->vocab_size) h->segments *= 2;
   h->seg_len = ((c->vocab_size + h->segments - 1) / h->segments + 3) / 4 * 4;
   h->segments = (c->vocab_size + h->seg_len - 1) / h->seg_len;
-  if ((e = hipMalloc(&h->d_workspace, sizeof(unsigned long long) * c->batch_size * h->segments * k)) != hipSuccess)
+  if ((e = hipMalloc(&h->d_workspace, sizeof(unsigned long long) * c->batch_size * h->segments * kSlots)) != hipSuccess)
     return bail(MI355_SAMPLER_RESOURCE_EXHAUSTED, "candidate workspace", e);
   if (c->host_io) {
     const size_t B = c->batch_size, V = c->vocab_size, K = std::min<size_t>(k, V);
