@@ -261,7 +261,9 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: block addresses stay scalar
   const int n = lane & 15, g = lane >> 4;
-  const int split = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z;
+  // Partitions vary slowest in dispatch order: with ragged lengths the empty ones
+  // (sequences shorter than the longest) then come last instead of between the full ones.
+  const int split = blockIdx.z, kvh = blockIdx.y, item = blockIdx.x;
   const int li = item / a.batch, b = item - li * a.batch;
   const int layer = a.layer_begin + li;
   const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
@@ -414,7 +416,7 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
 template <int KV, int IO, int D, int NW>
 hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int items = a.n_layers * a.batch;
-  const dim3 grid(a.num_splits, a.geom.hkv, items);
+  const dim3 grid(items, a.geom.hkv, a.num_splits);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
   // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
