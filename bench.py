@@ -38,8 +38,8 @@ METRIC = "decode-attn HBM GB/s (% of 8 TB/s) + prefill-attn TFLOP/s, Gemma3n-E2B
 # HBM bytes per decode launch of the headline workload, from
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script, each
 # scaled by what the same counter reads for a plain copy of known size
-# (profiles/bench_default_hbm_traffic.txt): 123,414 KiB x 2.0 fetched + 3,960 KiB x 1.0 written.
-MEASURED_TRAFFIC_BYTES = 256806912
+# (profiles/bench_default_hbm_traffic.txt): 123,054 KiB x 2.0 fetched + 3,900 KiB x 1.0 written.
+MEASURED_TRAFFIC_BYTES = 256008192
 
 
 def log(*a):
