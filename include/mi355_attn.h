@@ -238,6 +238,13 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      (the only path for fp32 and int8 caches)
  *   "prefill_workgroups" upper bound of the persistent workgroups of the prefill
  *                      kernel, 0 (default) = one per compute unit
+ *   "prefill_key_split" -1 (default): a prefill launch with fewer work items than
+ *                      three quarters of the compute units (a single layer, say) cuts
+ *                      the key range of its tiles into up to 8 work items each and
+ *                      merges their results in a second kernel; the fp32 parts go to a
+ *                      workspace allocated on first use, [layers][rows][heads][parts]
+ *                      x (head_dim + 2) floats, at most 258 MiB (else no split).
+ *                      0: never; n > 0: n key blocks (of 32 keys) per work item
  *   "prefill_bf16_single_p" 0 (default): a bf16 prefill feeds each probability to
  *                      the P.V product as a high and a low bf16 part, which keeps the
  *                      result within the output format's own rounding; 1: one bf16

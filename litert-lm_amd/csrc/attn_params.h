@@ -136,6 +136,13 @@ struct PrefillArgs {
   const int32_t* host_window;  // host copy of layer_window (for the ordering), may be null
   int32_t use_order;
   int32_t single_p;  // bf16: probabilities enter P.V as one bf16 operand (faster, ~1.5e-3 L2 error) instead of two
+  // Key split (launches with fewer work items than compute units): a work item covers at most kchunk
+  // key blocks of its tile, tiles with more blocks are cut into up to smax items whose unnormalised
+  // fp32 accumulators and (max, sum) pairs go to ws_acc / ws_ml, [layer][row][head][smax] x head_dim
+  // and x 2 floats, and prefill_merge_kernel combines them. kchunk == 0: off.
+  int32_t kchunk, smax;
+  float* ws_acc;
+  float* ws_ml;
   uint16_t unit_order[128];
 };
 constexpr int kPrefillQueues = 2;                     // ticket queues; workgroup k draws from queue k % 2 first

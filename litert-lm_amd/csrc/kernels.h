@@ -22,6 +22,18 @@ hipError_t launch_decode(const DecodeArgs& args, int kv_dtype, int io_dtype, con
 
 bool prefill_supported(int kv_dtype, int io_dtype, int head_dim);
 
+// Key split of a prefill launch (PrefillArgs::kchunk / smax): none (kchunk 0) unless the launch has
+// fewer work items than three quarters of the compute units; then at most 8 items per tile of at
+// least 4 key blocks each. option > 0 forces that many key blocks per item (tests), option 0 is off,
+// option < 0 the rule above. Reads n_layers, geom.hkv, group, n, q_pos0, layer_begin, host_window.
+struct PrefillSplit {
+  int kchunk = 0, smax = 1;
+  size_t rows = 0;  // rows of the workspace: n_layers * n * hq * smax
+};
+PrefillSplit plan_prefill_split(const PrefillArgs& args, int option);
+
+// With args.kchunk > 0 the merge kernel follows the attention kernel (ev1 then marks the end of the
+// attention kernel alone).
 hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, hipStream_t stream,
                           hipEvent_t ev0, hipEvent_t ev1);
 

@@ -71,6 +71,10 @@ struct mi355_attn {
   float* scales = nullptr;
   int32_t* d_window = nullptr;
   int32_t* d_sched = nullptr;  // prefill work-queue counters
+  float* d_pf_acc = nullptr;   // prefill key split: parts of split tiles, allocated on first use
+  float* d_pf_ml = nullptr;
+  size_t pf_rows = 0;          // rows (of head_dim / of 2 floats) the two hold
+  int prefill_key_split = -1;  // < 0 by rule, 0 off, > 0 key blocks per work item
   // the step before attention: per-layer constants in HBM and what is switched on
   struct LayerTransform {
     bool set = false, rope = false, norm_q = false, norm_k = false, norm_v = false, q_scaled = false, k_scaled = false;
@@ -324,6 +328,28 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.max_workgroups = h->prefill_workgroups;
     a.single_p = h->bf16_single_p ? 1 : 0;
     a.host_window = h->window.data();
+    PrefillSplit split = plan_prefill_split(a, h->prefill_key_split);
+    constexpr size_t kSplitRowsMax = (size_t)256 << 10;  // 256 Ki rows = 258 MiB at head_dim 256
+    if (split.kchunk > 0 && split.rows > kSplitRowsMax && h->prefill_key_split < 0) split = PrefillSplit{};
+    if (split.kchunk > 0) {
+      if (split.rows > kSplitRowsMax)
+        return fail(error_msg, MI355_ATTN_RESOURCE_EXHAUSTED, "prefill_key_split=%d needs %zu workspace rows (limit %zu)",
+                    h->prefill_key_split, split.rows, kSplitRowsMax);
+      if (h->pf_rows < split.rows) {
+        HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+        if (h->d_pf_acc) HIP_OR_RETURN(hipFree(h->d_pf_acc));
+        if (h->d_pf_ml) HIP_OR_RETURN(hipFree(h->d_pf_ml));
+        h->d_pf_acc = h->d_pf_ml = nullptr;
+        h->pf_rows = 0;
+        HIP_OR_RETURN(hipMalloc(&h->d_pf_acc, split.rows * h->cfg.head_dim * sizeof(float)));
+        HIP_OR_RETURN(hipMalloc(&h->d_pf_ml, split.rows * 2 * sizeof(float)));
+        h->pf_rows = split.rows;
+      }
+      a.kchunk = split.kchunk;
+      a.smax = split.smax;
+      a.ws_acc = h->d_pf_acc;
+      a.ws_ml = h->d_pf_ml;
+    }
     HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
   } else {
     // Row-wise path (fp32 and int8 caches): every query row is one decode item
@@ -493,6 +519,8 @@ void mi355_attn_destroy(mi355_attn* h) {
   if (h->scales) (void)hipFree(h->scales);
   if (h->d_window) (void)hipFree(h->d_window);
   if (h->d_sched) (void)hipFree(h->d_sched);
+  if (h->d_pf_acc) (void)hipFree(h->d_pf_acc);
+  if (h->d_pf_ml) (void)hipFree(h->d_pf_ml);
   if (h->d_transform) (void)hipFree(h->d_transform);
   if (h->ws_acc) (void)hipFree(h->ws_acc);
   if (h->ws_ml) (void)hipFree(h->ws_ml);
@@ -743,6 +771,9 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   } else if (!strcmp(name, "prefill_workgroups")) {
     if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_workgroups = value;
+  } else if (!strcmp(name, "prefill_key_split")) {
+    if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;
+    h->prefill_key_split = value;
   } else if (!strcmp(name, "prefill_bf16_single_p")) {
     h->bf16_single_p = value != 0;
   } else {

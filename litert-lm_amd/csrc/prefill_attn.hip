@@ -144,6 +144,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int tiles = (a.n + kStretch * PT - 1) / (kStretch * PT);
   const int home = blockIdx.x & (kPrefillQueues - 1);
   int tried = 0;  // queues this workgroup has found empty (kept by thread 0)
+  const int smax = a.kchunk > 0 ? a.smax : 1;  // work items per tile (key split), some of them empty
   const float softcap = a.softcap;  // CAP: > 0, scores go through softcap * tanh(score / softcap)
   const float c = CAP ? 1.f : a.scale * kLog2e;
   const int pos_end = a.q_pos0 + a.n;                // one past the last query position
@@ -153,15 +154,50 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int v_off = (n >> 4) * 1024 + hh * 256 + (n & 15) * 16;
   constexpr int kAhead = 4;  // K operand reads in flight ahead of their MFMAs
 
+  // A ticket of a queue with qcnt units is (tile, part, unit), tile-major: a
+  // queue's longest key loops first. Key blocks of a tile: from the first one the
+  // window of its first row reaches to the one holding the diagonal of its last
+  // valid row; part p of a split tile covers blocks [p * kchunk, (p + 1) * kchunk)
+  // of those.
+  struct Item { int li, kvh, hb, tile, part, layer, window, wg_pos0, kb_lo, nblk_tile; };
+  auto item_of = [&](int qx, int ticket) {
+    Item it;
+    const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
+    const int per_tile = qcnt * smax;
+    const int ti = ticket / per_tile, r2 = ticket - ti * per_tile;
+    it.part = r2 / qcnt;
+    const int slot = qx + kPrefillQueues * (r2 - it.part * qcnt);
+    const int u = a.use_order ? a.unit_order[slot] : slot;
+    it.li = u / per_layer;
+    const int rem = u - it.li * per_layer;
+    it.kvh = rem / hblocks;
+    it.hb = rem - it.kvh * hblocks;
+    it.tile = tiles - 1 - ti;
+    it.layer = a.layer_begin + it.li;
+    it.window = a.layer_window[it.layer];
+    it.wg_pos0 = a.q_pos0 + it.tile * (kStretch * PT);  // first position of the workgroup
+    const int last_pos = min(it.wg_pos0 + kStretch * PT, pos_end) - 1;
+    it.kb_lo = 0;
+    if (it.window > 0 && it.wg_pos0 - it.window + 1 > 0) it.kb_lo = (it.wg_pos0 - it.window + 1) / kKeysPerBlock;
+    it.nblk_tile = last_pos / kKeysPerBlock - it.kb_lo + 1;
+    return it;
+  };
+
   for (;;) {
   if (tid == 0) {
     int x = 0, t = -1;
     while (tried < kPrefillQueues) {
       x = (home + tried) & (kPrefillQueues - 1);
-      const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;  // units x, x + 8, ...
+      const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;  // units x, x + 2, ...
       if (cnt > 0) {
         t = atomicAdd(a.sched + x, 1);
-        if (t < cnt * tiles) break;
+        if (t < cnt * tiles * smax) {
+          if (smax == 1) break;
+          const Item it = item_of(x, t);
+          if (it.part * a.kchunk < it.nblk_tile) break;
+          t = -1;  // a part past the tile's last block: draw again from the same queue
+          continue;
+        }
         t = -1;
       }
       ++tried;
@@ -174,30 +210,20 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int qx = __builtin_amdgcn_readfirstlane(sm_ticket[0]);
   const int ticket = __builtin_amdgcn_readfirstlane(sm_ticket[1]);
   if (ticket < 0) break;  // every queue is empty: the only exit, reached by all workgroups
-  const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
-  const int ti = ticket / qcnt, ui = ticket - ti * qcnt;  // stretch-major: a queue's longest loops first
-  const int slot = qx + kPrefillQueues * ui;
-  const int u = a.use_order ? a.unit_order[slot] : slot;
-  const int li = u / per_layer, rem = u - li * per_layer;
-  const int kvh = rem / hblocks, hb = rem - kvh * hblocks;
-  const int tile = tiles - 1 - ti;
-  const int layer = a.layer_begin + li;
-  const int window = a.layer_window[layer];
+  const Item it = item_of(qx, ticket);
+  const int li = it.li, kvh = it.kvh, hb = it.hb, layer = it.layer, window = it.window, wg_pos0 = it.wg_pos0;
   const int head = kvh * a.group + hb * HPB + (wave % HPB);
-  const int wg_pos0 = a.q_pos0 + tile * (kStretch * PT);  // first position of the workgroup
   const int my_pos0 = wg_pos0 + (wave / HPB) * kStretch;  // first position of this wave's stretch
   const int my_pos = my_pos0 + n;
 
   const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
   const uint8_t* vplane = kplane + a.geom.plane_bytes;
 
-  // Key blocks the workgroup walks: from the first one the window of its first
-  // row reaches to the one holding the diagonal of its last valid row. Every
-  // wave walks all of them (blocks outside a tile's range are masked).
-  const int last_pos = min(wg_pos0 + kStretch * PT, pos_end) - 1;
-  int kb_lo = 0;
-  if (window > 0 && wg_pos0 - window + 1 > 0) kb_lo = (wg_pos0 - window + 1) / kKeysPerBlock;
-  const int nblk = last_pos / kKeysPerBlock - kb_lo + 1;
+  // Key blocks the workgroup walks (every wave walks all of them; blocks outside
+  // a row's range are masked): the tile's, or this part of them.
+  const bool split_tile = smax > 1 && it.nblk_tile > a.kchunk;
+  const int kb_lo = it.kb_lo + (smax > 1 ? it.part * a.kchunk : 0);
+  const int nblk = smax > 1 ? min(a.kchunk, it.nblk_tile - it.part * a.kchunk) : it.nblk_tile;
 
   // A K or V block travels HBM/L2 -> LDS without touching registers: every
   // wave issues kXfers of the 16 wave-wide 1 KiB transfers of a block; the data
@@ -500,7 +526,40 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   // wave has its own patch, rows padded to 528 bytes against bank conflicts) and
   // leave as whole 512-byte rows, two per store instruction.
   lds_barrier();  // every wave is done with the last V block
-  {
+  if (split_tile) {
+    // A part of a split tile: the unnormalised accumulators (fp32) and the row's
+    // (reference max, sum) go to the workspace, again as whole rows through LDS.
+    // The patches of waves 2 and 3 start behind the ticket words, which thread 0
+    // may rewrite for the next item while they are still being read.
+    constexpr int kRowStrideF = 4 * D + 16;
+    static_assert(2 * (kStretch * kRowStrideF) <= (kStages + kStages - 1) * kBlockBytes, "patches 0, 1 before the ticket");
+    uint8_t* const patch = smem + wave * (kStretch * kRowStrideF) + (wave >= 2 ? 16384 : 0);
+    const float l_tot = wave_xor_add(l_run0, 32);
+#pragma unroll
+    for (int dp = 0; dp < NDP; ++dp) {
+#pragma unroll
+      for (int aa = 0; aa < 4; ++aa) {
+        f4 o;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) o[b] = acc0[dp][4 * aa + b];
+        *reinterpret_cast<f4*>(patch + n * kRowStrideF + (32 * dp + 8 * aa + 4 * hh) * 4) = o;
+      }
+    }
+    const int row_base = my_pos0 - a.q_pos0;
+    if (hh == 0 && row_base + n < a.n) {
+      const int64_t slot = (((int64_t)li * a.n + row_base + n) * a.hq + head) * smax + it.part;
+      *reinterpret_cast<float2*>(a.ws_ml + slot * 2) = float2{m_run0, l_tot};
+    }
+#pragma unroll 4
+    for (int r = 0; r < kStretch; ++r) {
+      const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStrideF + lane * 16);
+      const int row = row_base + r;
+      if (row < a.n) {
+        const int64_t slot = (((int64_t)li * a.n + row) * a.hq + head) * smax + it.part;
+        *reinterpret_cast<u4*>(a.ws_acc + slot * D + lane * 4) = w;
+      }
+    }
+  } else {
     constexpr int kRowStride = 2 * D + 16;
     uint8_t* const patch = smem + wave * (kStretch * kRowStride);
     const float l_tot = wave_xor_add(l_run0, 32);
@@ -538,6 +597,34 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     if (done == (int)gridDim.x - 1)
       for (int i = 0; i < kPrefillSchedInts; ++i) atomicExch(a.sched + i, 0);
   }
+}
+
+// Combines the parts of split tiles: grid (query head, row, layer), one thread
+// per channel. Rows of tiles that were not split have been written by the
+// attention kernel itself.
+template <int DT, int D>
+__global__ void __launch_bounds__(D) prefill_merge_kernel(const PrefillArgs a, int rows_per_tile) {
+  using elem_t = typename El<DT>::type;
+  const int head = blockIdx.x, row = blockIdx.y, li = blockIdx.z, d = threadIdx.x;
+  const int window = a.layer_window[a.layer_begin + li];
+  const int wg_pos0 = a.q_pos0 + (row / rows_per_tile) * rows_per_tile;
+  const int last_pos = min(wg_pos0 + rows_per_tile, a.q_pos0 + a.n) - 1;
+  int kb_lo = 0;
+  if (window > 0 && wg_pos0 - window + 1 > 0) kb_lo = (wg_pos0 - window + 1) / kKeysPerBlock;
+  const int nblk = last_pos / kKeysPerBlock - kb_lo + 1;
+  if (nblk <= a.kchunk) return;
+  const int parts = (nblk + a.kchunk - 1) / a.kchunk;
+  const int64_t slot0 = (((int64_t)li * a.n + row) * a.hq + head) * a.smax;
+  float M = -INFINITY;
+  for (int p = 0; p < parts; ++p) M = fmaxf(M, a.ws_ml[(slot0 + p) * 2]);
+  float A = 0.f, L = 0.f;
+  for (int p = 0; p < parts; ++p) {
+    const float m = a.ws_ml[(slot0 + p) * 2];
+    const float wgt = m == -INFINITY ? 0.f : fast_exp2(m - M);  // (a part none of whose keys the row sees)
+    A += wgt * a.ws_acc[(slot0 + p) * D + d];
+    L += wgt * a.ws_ml[(slot0 + p) * 2 + 1];
+  }
+  reinterpret_cast<elem_t*>(a.out)[(((int64_t)li * a.n + row) * a.hq + head) * D + d] = (elem_t)(L > 0.f ? A / L : 0.f);
 }
 
 template <int DT, int D, int HPB, bool CAP, bool SPLITP>
@@ -605,15 +692,59 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
     for (int u = 0; u < units; ++u) b.unit_order[u] = (uint16_t)order[u];
     b.use_order = 1;
   }
-  int wgs = items < cus ? items : cus;
+  const long all_items = (long)items * (a.kchunk > 0 ? a.smax : 1);  // (some of them empty when tiles are split)
+  int wgs = all_items < cus ? (int)all_items : cus;
   if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
   const dim3 grid(wgs, 1, 1);
-  if (hpb == 4) return launch_hpb<DT, D, 4>(b, grid, stream, ev0, ev1);
-  if (hpb == 2) return launch_hpb<DT, D, 2>(b, grid, stream, ev0, ev1);
-  return launch_hpb<DT, D, 1>(b, grid, stream, ev0, ev1);
+  hipError_t err = hpb == 4   ? launch_hpb<DT, D, 4>(b, grid, stream, ev0, ev1)
+                   : hpb == 2 ? launch_hpb<DT, D, 2>(b, grid, stream, ev0, ev1)
+                              : launch_hpb<DT, D, 1>(b, grid, stream, ev0, ev1);
+  if (err != hipSuccess || a.kchunk <= 0) return err;
+  hipLaunchKernelGGL((prefill_merge_kernel<DT, D>), dim3(a.hq, a.n, a.n_layers), dim3(D), 0, stream, b, kStretch * pt);
+  return hipGetLastError();
 }
 
 }  // namespace
+
+PrefillSplit plan_prefill_split(const PrefillArgs& a, int option) {
+  PrefillSplit out;
+  if (option == 0 || !a.host_window) return out;
+  const int G = a.group;
+  const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
+  const int rows_per_tile = kStretch * (4 / hpb);
+  const int tiles = (a.n + rows_per_tile - 1) / rows_per_tile;
+  const long items = (long)a.n_layers * a.geom.hkv * (G / hpb) * tiles;
+  int max_nblk = 1;
+  for (int li = 0; li < a.n_layers; ++li) {
+    const int w = a.host_window[a.layer_begin + li];
+    for (int t = 0; t < tiles; ++t) {
+      const int p0 = a.q_pos0 + t * rows_per_tile;
+      const int last = std::min(p0 + rows_per_tile, a.q_pos0 + a.n) - 1;
+      const int lo = (w > 0 && p0 - w + 1 > 0) ? (p0 - w + 1) / kKeysPerBlock : 0;
+      max_nblk = std::max(max_nblk, last / kKeysPerBlock - lo + 1);
+    }
+  }
+  int kchunk;
+  if (option > 0) {
+    kchunk = option;
+  } else {
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      return out;
+    if (items * 4 >= (long)cus * 3) return out;
+    int want = (int)std::min<long>(8, (cus + items - 1) / items);
+    want = std::min(want, max_nblk / 4);  // at least 4 key blocks per item
+    if (want <= 1) return out;
+    kchunk = (max_nblk + want - 1) / want;
+  }
+  const int smax = (max_nblk + kchunk - 1) / kchunk;
+  if (smax <= 1) return out;
+  out.kchunk = kchunk;
+  out.smax = smax;
+  out.rows = (size_t)a.n_layers * a.n * a.hq * smax;
+  return out;
+}
 
 bool prefill_supported(int kv_dtype, int io_dtype, int head_dim) {
   return head_dim == 256 && kv_dtype == io_dtype && (kv_dtype == kF16 || kv_dtype == kBF16);

@@ -336,6 +336,10 @@ def test_prefill_chunked_equals_one_shot_and_layers_call():
             kd, _ = dev(gen(72 + layer, 1024, 1, D), A.BF16)
             vd, _ = dev(gen(75 + layer, 1024, 1, D), A.BF16)
             at.kv_append(layer, 0, 0, kd, vd)
+        # (launches this small would cut their key ranges into parts, one layer into more than two,
+        # which changes the summation order: switched off for the bit-exact comparison; covered by
+        # test_prefill_key_split_*)
+        at.set_option("prefill_key_split", 0)
         one = torch.empty_like(qd)
         at.prefill(0, 0, 0, 1024, qd, one, n_layers=nl)
         per = torch.empty_like(qd)
@@ -350,16 +354,88 @@ def test_prefill_chunked_equals_one_shot_and_layers_call():
         assert orc.rel_err(two.float().cpu().numpy(), one.float().cpu().numpy()) < TOL[A.BF16]
 
 
+@pytest.mark.parametrize("dt", [A.BF16, A.F16])
+@pytest.mark.parametrize("hq,hkv,kchunk", [(4, 1, 1), (4, 1, 3), (8, 2, 2), (3, 1, 5), (2, 2, 4)])
+def test_prefill_key_split_matches_oracle(dt, hq, hkv, kchunk):
+    """Tiles cut into work items of `kchunk` key blocks whose parts a second kernel merges: global and
+    windowed layers, ragged ends, a later chunk of a longer context, rows that see no key of a part
+    (causal: the early rows of a tile and its last part; window: the late rows and its first part)."""
+    windows = [0, 40, 1, 33, 200]
+    L = 700
+    with make(len(windows), hq, hkv, L, 1, dt, layer_window=windows) as at:
+        at.set_option("prefill_key_split", kchunk)
+        k, v = gen(261, L, hkv, D), gen(262, L, hkv, D)
+        for layer, w in enumerate(windows):
+            kr, vr = fill_seq(at, dt, layer, 0, k, v)
+            for q_pos0, n in ((0, 1), (0, 33), (0, 257), (129, 200), (300, 400), (699, 1)):
+                q = gen(3000 + n + q_pos0, n, hq, D)
+                err, out = run_prefill(at, dt, q, kr, vr, q_pos0, w, layer=layer)
+                assert err < TOL[dt], (hq, hkv, kchunk, w, q_pos0, n, err)
+        # several layers in one launch, cut the same way
+        nl = len(windows)
+        qd, qr = dev(gen(271, nl, 300, hq, D), dt)
+        out = torch.empty_like(qd)
+        at.prefill(0, 0, 400, 300, qd, out, n_layers=nl)
+        torch.cuda.synchronize()
+        for layer, w in enumerate(windows):
+            ref = c_oracle.sdpa_f64(qr[layer], kr, vr, D ** -0.5, q_pos0=400, window=w, kv_len=700)
+            err = err_of(out[layer].float().cpu().numpy(), ref, dt)
+            assert err < TOL[dt], ("layers", hq, hkv, kchunk, w, err)
+    say(f"prefill key split dt={dt} hq={hq} hkv={hkv} kchunk={kchunk}: ok")
+
+
+def test_prefill_key_split_by_rule_softcap_and_limits():
+    # by rule (the default): one 1024-token global layer of config 2 has 32 tiles for 256 compute units
+    seed = orc.SEED_BASE + 1
+    with make(1, 4, 1, 1024, 1, A.BF16, layer_window=[0]) as at:
+        q = gen(seed + 1, 1024, 4, D)
+        kr, vr = fill_seq(at, A.BF16, 0, 0, gen(seed + 11, 1024, 1, D), gen(seed + 21, 1024, 1, D))
+        err, split = run_prefill(at, A.BF16, q, kr, vr, 0, 0)
+        assert err < TOL[A.BF16]
+        at.set_option("prefill_key_split", 0)
+        err0, whole = run_prefill(at, A.BF16, q, kr, vr, 0, 0)
+        assert err0 < TOL[A.BF16]
+        assert not torch.equal(split, whole)  # the rule did cut this launch: another summation order
+        say(f"key split by rule: rel_err {err:.3e}, unsplit {err0:.3e}")
+    # soft cap (the visibility test then follows the cap) and a scale of its own
+    with make(1, 4, 2, 300, 1, A.F16, layer_window=[70], scale=0.09, softcap=5.0) as at:
+        at.set_option("prefill_key_split", 2)
+        kr, vr = fill_seq(at, A.F16, 0, 0, gen(281, 300, 2, D), gen(282, 300, 2, D))
+        qd, qr = dev(gen(283, 250, 4, D), A.F16)
+        out = torch.empty_like(qd)
+        at.prefill(0, 0, 50, 250, qd, out)
+        torch.cuda.synchronize()
+        ref = c_oracle.sdpa_f64(qr, kr, vr, 0.09, q_pos0=50, window=70, softcap=5.0, kv_len=300)
+        err = err_of(out.float().cpu().numpy(), ref, A.F16)
+        say(f"key split with soft cap: rel_err {err:.3e}")
+        assert err < TOL[A.F16]
+    # a forced split whose parts would not fit the workspace limit is refused, not shrunk
+    with make(1, 8, 2, 8192, 1, A.F16) as at:
+        at.set_option("prefill_key_split", 1)
+        kd, _ = dev(np.zeros((8192, 2, D), np.float32), A.F16)
+        at.kv_append(0, 0, 0, kd, kd)
+        qd, _ = dev(np.zeros((8192, 8, D), np.float32), A.F16)
+        out = torch.empty_like(qd)
+        with pytest.raises(A.AttnError) as ei:
+            at.prefill(0, 0, 0, 8192, qd, out)
+        assert ei.value.code == A.RESOURCE_EXHAUSTED
+    with make(1, 4, 1, 64, 1, A.F16) as at:
+        with pytest.raises(A.AttnError):
+            at.set_option("prefill_key_split", -2)
+
+
 @pytest.mark.parametrize("dt", [A.F16, A.BF16])
-@pytest.mark.parametrize("hq,hkv", [(4, 1), (8, 4), (3, 1)])
-def test_prefill_many_work_items_per_workgroup(dt, hq, hkv):
+@pytest.mark.parametrize("hq,hkv,key_split", [(4, 1, 0), (8, 4, 0), (3, 1, 0), (4, 1, 3), (8, 4, 2)])
+def test_prefill_many_work_items_per_workgroup(dt, hq, hkv, key_split):
     """Few persistent workgroups walking many work items each (what one launch over 26 layers does on
-    the full chip): the hand-over between items -- tickets, rings, query rows, output rows -- must not
-    depend on how many workgroups share the queue. Short and long items, ragged ends, local and global
-    layers, a later chunk."""
+    the full chip): the hand-over between items -- tickets, rings, query rows, output rows or parts of
+    split tiles -- must not depend on how many workgroups share the queue. Short and long items,
+    ragged ends, local and global layers, a later chunk; whole tiles and tiles cut every `key_split`
+    key blocks (the same cut in every launch, so the bits must agree)."""
     nl, n, pos0 = 5, 333, 160
     windows = [0, 70, 0, 512, 33]
     with make(nl, hq, hkv, pos0 + n, 1, dt, layer_window=windows) as at:
+        at.set_option("prefill_key_split", key_split)
         qd, _ = dev(gen(91, nl, n, hq, D), dt)
         for layer in range(nl):
             kd, _ = dev(gen(92 + layer, pos0 + n, hkv, D), dt)
