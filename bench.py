@@ -172,6 +172,14 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, sin
     def step1(i):
         at.prefill(5, 0, 0, n, q[5], out[5])  # one global layer
     lat1 = time_steps(torch, step1, 50, 5)
+
+    def step_layers(i):  # the way an executor calls it: one launch per layer, in turn
+        for layer in range(layers):
+            at.prefill(layer, 0, 0, n, q[layer], out[layer])
+    per_layer = time_steps(torch, step_layers, 10, 2)
+    at.set_option("prefill_key_split", 0)
+    lat1_whole = time_steps(torch, step1, 50, 5)
+    per_layer_whole = time_steps(torch, step_layers, 10, 2)
     at.close()
     return {"workload": f"C2: 26 layers x 1024 tokens, Hq4/Hkv1, {'fp16' if half else 'bf16'}, "
                         "22 local(W=512)+4 global, one launch",
@@ -179,6 +187,8 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, sin
             "kernel_TFLOPs": flops / (kms * 1e-3) / 1e12,
             "frac_of_mfma_peak": flops / (kms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
             "tokens_per_s": n / sec, "single_global_layer_ms": lat1 * 1e3,
+            "single_global_layer_unsplit_ms": lat1_whole * 1e3,
+            "layer_by_layer_ms": per_layer * 1e3, "layer_by_layer_unsplit_ms": per_layer_whole * 1e3,
             "dense_counted_TFLOPs": layers * 4 * hq * D * n * n / sec / 1e12}
 
 
@@ -407,6 +417,13 @@ def main():
             "workload": pre["workload"], "value": round(pre["TFLOPs"], 2), "unit": "TFLOP/s", "dtype": "bf16",
             "ms_per_step": round(pre["ms_per_step"], 4), "prefill_tokens_per_s": round(pre["tokens_per_s"], 1),
             "single_global_layer_ms": round(pre["single_global_layer_ms"], 4),
+            "layer_by_layer": {
+                "what": "the same 26 layers as 26 launches in turn (how an executor calls it); key ranges of a "
+                        "launch this small are cut into parts that a second kernel merges (option "
+                        "prefill_key_split, default by rule), *_unsplit: with that switched off",
+                "ms": round(pre["layer_by_layer_ms"], 4), "TFLOPs": round(pre["flops"] / pre["layer_by_layer_ms"] / 1e9, 2),
+                "unsplit_ms": round(pre["layer_by_layer_unsplit_ms"], 4),
+                "single_global_layer_unsplit_ms": round(pre["single_global_layer_unsplit_ms"], 4)},
             "dense_counted_TFLOPs": round(pre["dense_counted_TFLOPs"], 2),
             "roofline": {"kernel": "prefill_attn_kernel<bf16,256>", "bound": "mfma",
                          "achieved": round(pre["kernel_TFLOPs"], 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",

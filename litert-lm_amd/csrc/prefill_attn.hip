@@ -144,6 +144,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
   const int tiles = (a.n + kStretch * PT - 1) / (kStretch * PT);
   const int home = blockIdx.x & (kPrefillQueues - 1);
   int tried = 0;  // queues this workgroup has found empty (kept by thread 0)
+  bool first_draw = true;
   const int smax = a.kchunk > 0 ? a.smax : 1;  // work items per tile (key split), some of them empty
   const float softcap = a.softcap;  // CAP: > 0, scores go through softcap * tanh(score / softcap)
   const float c = CAP ? 1.f : a.scale * kLog2e;
@@ -190,7 +191,14 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
       x = (home + tried) & (kPrefillQueues - 1);
       const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;  // units x, x + 2, ...
       if (cnt > 0) {
-        t = atomicAdd(a.sched + x, 1);
+        // The first ticket of a workgroup on its home queue is its index among that
+        // queue's workgroups (hundreds of workgroups asking two counters at the
+        // start of a launch wait microseconds for each other); the counters hand
+        // out what follows.
+        const int home_wgs = ((int)gridDim.x - x + kPrefillQueues - 1) / kPrefillQueues;
+        if (first_draw && tried == 0) t = (int)blockIdx.x / kPrefillQueues;
+        else t = atomicAdd(a.sched + x, 1) + home_wgs;
+        first_draw = false;
         if (t < cnt * tiles * smax) {
           if (smax == 1) break;
           const Item it = item_of(x, t);
