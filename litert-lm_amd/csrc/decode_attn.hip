@@ -252,7 +252,13 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
   reinterpret_cast<io_t*>(a.out)[((int64_t)item * a.hq + head) * D + d] = (io_t)o;
 }
 
-template <int KV, int IO, int D, int NW>
+// INL: lengths, sequence ids and windows travel in the argument block (the host
+// knows: a.inline_items and n_layers <= kInlineLayers). Then everything in front
+// of the first loads is one round of scalar loads at addresses that depend on
+// the block index only. (With both sources behind one `cond ? a.inline_x[b] :
+// a.x[b]` the compiler selects a pointer and issues vector loads, one after the
+// other, and a wave spent 2 to 4 us before its first K/V load.)
+template <int KV, int IO, int D, int NW, bool INL>
 __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
   constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
@@ -261,24 +267,46 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: block addresses stay scalar
   const int n = lane & 15, g = lane >> 4;
-  // Partitions vary slowest in dispatch order: with ragged lengths the empty ones
-  // (sequences shorter than the longest) then come last instead of between the full ones.
-  const int split = blockIdx.z, kvh = blockIdx.y, item = blockIdx.x;
-  const int li = item / a.batch, b = item - li * a.batch;
-  const int layer = a.layer_begin + li;
-  const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
-  const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
-  const int window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
+  // Grid (sequence, layer, partition x KV head): partitions vary slowest in dispatch
+  // order, so with ragged lengths the empty ones (sequences shorter than the
+  // longest) come last instead of between the full ones.
+  const int b = blockIdx.x, li = blockIdx.y;
+  // What the code in front of the first K/V loads needs from the argument block is
+  // read here in one go (left alone, the compiler sinks each scalar load behind the
+  // branch that needs it: four dependent round trips instead of one).
+  int hkv = a.geom.hkv, batch = a.batch, layer_begin = a.layer_begin, max_seqs = a.geom.max_seqs;
+  int num_splits = a.num_splits, max_kv_len = a.max_kv_len;
+  int64_t plane_bytes = a.geom.plane_bytes;
+  const uint8_t* cache = a.cache;
+  int seq = 0, kv_len = 0, window = 0;
+  if constexpr (INL) {  // (addresses that depend on the block index only: the same round)
+    seq = a.inline_seq[b];
+    kv_len = a.inline_lens[b];
+    window = a.inline_window[li];
+  }
+  asm volatile("" : "+s"(hkv), "+s"(batch), "+s"(layer_begin), "+s"(max_seqs), "+s"(num_splits), "+s"(max_kv_len),
+               "+s"(plane_bytes), "+s"(cache), "+s"(seq), "+s"(kv_len), "+s"(window));
+  const int split = blockIdx.z / hkv, kvh = blockIdx.z - split * hkv;
+  const int item = li * batch + b;
+  const int layer = layer_begin + li;
+  if constexpr (!INL) {
+    seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
+    kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
+    window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
+  }
+  seq = __builtin_amdgcn_readfirstlane(seq);
+  kv_len = __builtin_amdgcn_readfirstlane(kv_len);
+  window = __builtin_amdgcn_readfirstlane(window);
   int vlo, start;
   decode_visible_range(kv_len, window, &vlo, &start);
-  const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
+  const int per = decode_partition_tokens(max_kv_len, window, num_splits);
   const int p_lo = start + split * per;
   const int p_hi = min(kv_len, p_lo + per);
   if (p_lo >= p_hi) return;  // empty partition: uniform over the workgroup
 
-  const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, seq, kvh, 0);
-  const __amdgpu_buffer_rsrc_t krsrc = plane_resource(kplane, a.geom.plane_bytes);
-  const __amdgpu_buffer_rsrc_t vrsrc = plane_resource(kplane + a.geom.plane_bytes, a.geom.plane_bytes);
+  const uint8_t* kplane = cache + ((((int64_t)layer * max_seqs + seq) * hkv + kvh) * 2) * plane_bytes;  // geom.plane_offset
+  const __amdgpu_buffer_rsrc_t krsrc = plane_resource(kplane, plane_bytes);
+  const __amdgpu_buffer_rsrc_t vrsrc = plane_resource(kplane + plane_bytes, plane_bytes);
   constexpr int kBlockBytes = 64 * D;
   const int blk_end = (p_hi + VB - 1) / VB;
   const int lane_off = lane * 16;
@@ -367,8 +395,40 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   float l_tot = wave_xor_add(l_run, 16);
   l_tot = wave_xor_add(l_tot, 32);
 
-  // Merge the waves through LDS: [NW][group][D] accumulators, then max, sum.
   const int G = a.group;
+  using io_t = typename IoT<IO>::type;
+  if constexpr (NW == 1) {
+    // One wave: nothing to merge. Lane (n, g) holds channels 16 * db + 4 * g .. + 3 of head n.
+    if (n < G) {
+      const int head = kvh * G + n;
+      if (a.num_splits == 1) {
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        io_t* orow = reinterpret_cast<io_t*>(a.out) + ((int64_t)item * a.hq + head) * D + 4 * g;
+        const float* vs = nullptr;
+        if constexpr (KV == kI8) vs = a.scales + a.geom.scale_offset(layer, seq, 1, kvh) + 4 * g;
+#pragma unroll
+        for (int db = 0; db < NL; ++db) {
+          io_t o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = acc[db][e] * inv;
+            if constexpr (KV == kI8) x *= vs[16 * db + e];
+            o[e] = (io_t)x;
+          }
+          if constexpr (sizeof(io_t) == 4) *reinterpret_cast<u4*>(orow + 16 * db) = *reinterpret_cast<const u4*>(o);
+          else *reinterpret_cast<u2*>(orow + 16 * db) = *reinterpret_cast<const u2*>(o);
+        }
+      } else {
+        const int64_t slot = ((int64_t)item * a.hq + head) * a.num_splits + split;
+        float* prow = a.ws_acc + slot * D + 4 * g;
+#pragma unroll
+        for (int db = 0; db < NL; ++db) *reinterpret_cast<f4*>(prow + 16 * db) = acc[db];
+        if (g == 0) *reinterpret_cast<float2*>(a.ws_ml + slot * 2) = float2{m_run, l_tot};
+      }
+    }
+    return;
+  }
+  // Merge the waves through LDS: [NW][group][D] accumulators, then max, sum.
   float* sm_acc = smem + NW * NQ * 64 * 4;  // behind the waves' Q slices
   float* sm_m = sm_acc + NW * G * D;
   float* sm_l = sm_m + NW * G;
@@ -383,7 +443,6 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   }
   __syncthreads();
 
-  using io_t = typename IoT<IO>::type;
   for (int e = threadIdx.x; e < G * D; e += NW * 64) {
     const int hn = e / D, d = e - hn * D;
     float M = -INFINITY;
@@ -413,19 +472,25 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   }
 }
 
-template <int KV, int IO, int D, int NW>
-hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+template <int KV, int IO, int D, int NW, bool INL>
+hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int items = a.n_layers * a.batch;
-  const dim3 grid(items, a.geom.hkv, a.num_splits);
+  const dim3 grid(a.batch, a.n_layers, a.num_splits * a.geom.hkv);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
   // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
   // begin and end timestamps, not the host-side launch latency around it.
-  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
+  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || a.num_splits == 1) return err;
   hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D>), dim3(a.hq, items), dim3(D), 0, stream, a);
   return hipGetLastError();
+}
+
+template <int KV, int IO, int D, int NW>
+hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  if (a.inline_items && a.n_layers <= kInlineLayers) return launch_inl<KV, IO, D, NW, true>(a, stream, ev0, ev1);
+  return launch_inl<KV, IO, D, NW, false>(a, stream, ev0, ev1);
 }
 
 template <int KV, int IO, int D>
