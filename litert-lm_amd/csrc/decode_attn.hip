@@ -195,6 +195,102 @@ __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)
   }
 }
 
+// One wave's share of a partition: blocks first, first + step, ... < blk_end of
+// the K / V planes behind krsrc / vrsrc, through the online softmax. Leaves the
+// reference max (exp2 domain), this lane's share of the sum (lane (n, g): head n,
+// tokens 4 g .. 4 g + 3 of every 16) and the unnormalised accumulators (channels
+// 16 * db + 4 * g .. + 3 of head n). Keys outside [vlo, p_hi) are masked.
+template <int KV, int IO, int D>
+__device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buffer_rsrc_t krsrc,
+                                              __amdgpu_buffer_rsrc_t vrsrc, int first, int blk_end, int step, int vlo,
+                                              int p_hi, u4* sm_q, int item, int kvh, int seq, int layer, int lane,
+                                              float& m_run, float& l_run, f4 (&acc)[D / 16]) {
+  constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
+  constexpr int kBlockBytes = 64 * D;
+  const int g = lane >> 4;
+  const int lane_off = lane * 16;
+  // Rolling prefetch: the K registers are refilled with the next block as soon
+  // as the QK^T product has consumed them, the V registers right after P.V, so
+  // 16 to 32 KiB per wave are in flight while it computes.
+  u4 kreg[NL], vreg[NL];
+  int blk = __builtin_amdgcn_readfirstlane(first);
+  if (blk < blk_end) {
+    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
+    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
+  }
+  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, lane);
+
+  m_run = -INFINITY;
+  l_run = 0.f;
+#pragma unroll
+  for (int i = 0; i < NL; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+  const float sc = a.scale, softcap = a.softcap;
+
+  while (blk < blk_end) {
+    // The index is made opaque so the Q reads stay inside the loop: hoisted
+    // they would occupy 32 to 64 registers for the whole kernel.
+    int qi = lane;
+    asm volatile("" : "+v"(qi));
+    f4 s[NT];
+    qk_block<KV, D>(kreg, sm_q, qi, s);
+    const int nxt = blk + step;
+    if (nxt < blk_end) load_plane_block<D>(kreg, krsrc, nxt * kBlockBytes, lane_off);
+
+    // scores in the exp2 domain; soft-capping and the range mask are uniform
+    // branches taken only by the layers / boundary blocks that need them
+    if (softcap > 0.f) {
+      const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
+#pragma unroll
+      for (int T = 0; T < NT; ++T)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[T][i] = cap2 * fast_tanh(s[T][i] * inv_cap);
+    } else {
+      const float sc2 = sc * kLog2e;
+#pragma unroll
+      for (int T = 0; T < NT; ++T) s[T] *= sc2;
+    }
+    if (blk * VB < vlo || (blk + 1) * VB > p_hi) {
+      const int tok0 = blk * VB + 4 * g;
+#pragma unroll
+      for (int T = 0; T < NT; ++T)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = tok0 + 16 * T + i;
+          s[T][i] = (tok >= vlo && tok < p_hi) ? s[T][i] : -INFINITY;
+        }
+    }
+    float bm = -INFINITY;
+#pragma unroll
+    for (int T = 0; T < NT; ++T)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[T][i]);
+    bm = wave_xor_max(bm, 16);
+    bm = wave_xor_max(bm, 32);
+    const float m_new = fmaxf(m_run, bm);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_use);
+    float lsum = 0.f;
+#pragma unroll
+    for (int T = 0; T < NT; ++T) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = fast_exp2(s[T][i] - m_use);
+        s[T][i] = pv;
+        lsum += pv;
+      }
+    }
+    l_run = l_run * alpha + lsum;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) acc[i] *= alpha;
+    pv_block<KV, D>(vreg, s, acc);
+    if (nxt < blk_end) load_plane_block<D>(vreg, vrsrc, nxt * kBlockBytes, lane_off);
+    blk = nxt;
+  }
+
+  // The four lanes (g = 0..3) of a head each summed their own tokens.
+}
+
 // Log-sum-exp merge of the split-KV partials: grid (query head, item), one
 // thread per channel. A separate launch because partials written by workgroups
 // on other XCDs are only guaranteed visible across a kernel boundary; an
@@ -260,7 +356,7 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
 // other, and a wave spent 2 to 4 us before its first K/V load.)
 template <int KV, int IO, int D, int NW, bool INL>
 __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
-  constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
+  constexpr int VB = KvT<KV>::VB, NL = D / 16;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   extern __shared__ float smem[];
 
@@ -307,91 +403,13 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   const uint8_t* kplane = cache + ((((int64_t)layer * max_seqs + seq) * hkv + kvh) * 2) * plane_bytes;  // geom.plane_offset
   const __amdgpu_buffer_rsrc_t krsrc = plane_resource(kplane, plane_bytes);
   const __amdgpu_buffer_rsrc_t vrsrc = plane_resource(kplane + plane_bytes, plane_bytes);
-  constexpr int kBlockBytes = 64 * D;
   const int blk_end = (p_hi + VB - 1) / VB;
-  const int lane_off = lane * 16;
 
-  // Rolling prefetch: the K registers are refilled with the next block as soon
-  // as the QK^T product has consumed them, the V registers right after P.V, so
-  // 16 to 32 KiB per wave are in flight while it computes.
-  u4 kreg[NL], vreg[NL];
-  int blk = __builtin_amdgcn_readfirstlane(p_lo / VB + wave);
-  if (blk < blk_end) {
-    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
-    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
-  }
   u4* sm_q = reinterpret_cast<u4*>(smem) + wave * (NQ * 64);
-  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, lane);
-
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run, l_run;
   f4 acc[NL];
-#pragma unroll
-  for (int i = 0; i < NL; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
-  const float sc = a.scale, softcap = a.softcap;
-
-  while (blk < blk_end) {
-    // The index is made opaque so the Q reads stay inside the loop: hoisted
-    // they would occupy 32 to 64 registers for the whole kernel.
-    int qi = lane;
-    asm volatile("" : "+v"(qi));
-    f4 s[NT];
-    qk_block<KV, D>(kreg, sm_q, qi, s);
-    const int nxt = blk + NW;
-    if (nxt < blk_end) load_plane_block<D>(kreg, krsrc, nxt * kBlockBytes, lane_off);
-
-    // scores in the exp2 domain; soft-capping and the range mask are uniform
-    // branches taken only by the layers / boundary blocks that need them
-    if (softcap > 0.f) {
-      const float inv_cap = sc / softcap, cap2 = softcap * kLog2e;
-#pragma unroll
-      for (int T = 0; T < NT; ++T)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s[T][i] = cap2 * fast_tanh(s[T][i] * inv_cap);
-    } else {
-      const float sc2 = sc * kLog2e;
-#pragma unroll
-      for (int T = 0; T < NT; ++T) s[T] *= sc2;
-    }
-    if (blk * VB < vlo || (blk + 1) * VB > p_hi) {
-      const int tok0 = blk * VB + 4 * g;
-#pragma unroll
-      for (int T = 0; T < NT; ++T)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = tok0 + 16 * T + i;
-          s[T][i] = (tok >= vlo && tok < p_hi) ? s[T][i] : -INFINITY;
-        }
-    }
-    float bm = -INFINITY;
-#pragma unroll
-    for (int T = 0; T < NT; ++T)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[T][i]);
-    bm = wave_xor_max(bm, 16);
-    bm = wave_xor_max(bm, 32);
-    const float m_new = fmaxf(m_run, bm);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
-    float lsum = 0.f;
-#pragma unroll
-    for (int T = 0; T < NT; ++T) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float pv = fast_exp2(s[T][i] - m_use);
-        s[T][i] = pv;
-        lsum += pv;
-      }
-    }
-    l_run = l_run * alpha + lsum;
-    m_run = m_new;
-#pragma unroll
-    for (int i = 0; i < NL; ++i) acc[i] *= alpha;
-    pv_block<KV, D>(vreg, s, acc);
-    if (nxt < blk_end) load_plane_block<D>(vreg, vrsrc, nxt * kBlockBytes, lane_off);
-    blk = nxt;
-  }
-
-  // The four lanes (g = 0..3) of a head each summed their own tokens.
+  stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, item, kvh, seq, layer, lane, m_run,
+                           l_run, acc);
   float l_tot = wave_xor_add(l_run, 16);
   l_tot = wave_xor_add(l_tot, 32);
 
