@@ -150,7 +150,7 @@ def prefill_flops(n, hq, window):
     return 4 * hq * D * pairs
 
 
-def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, single_p=False):
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, single_p=False, by_layer=False):
     hq, hkv = 4, 1
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
     stream = torch.cuda.current_stream().cuda_stream
@@ -176,10 +176,12 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, sin
     def step_layers(i):  # the way an executor calls it: one launch per layer, in turn
         for layer in range(layers):
             at.prefill(layer, 0, 0, n, q[layer], out[layer])
-    per_layer = time_steps(torch, step_layers, 10, 2)
-    at.set_option("prefill_key_split", 0)
-    lat1_whole = time_steps(torch, step1, 50, 5)
-    per_layer_whole = time_steps(torch, step_layers, 10, 2)
+    per_layer = lat1_whole = per_layer_whole = float("nan")
+    if by_layer:
+        per_layer = time_steps(torch, step_layers, 10, 2)
+        at.set_option("prefill_key_split", 0)
+        lat1_whole = time_steps(torch, step1, 50, 5)
+        per_layer_whole = time_steps(torch, step_layers, 10, 2)
     at.close()
     return {"workload": f"C2: 26 layers x 1024 tokens, Hq4/Hkv1, {'fp16' if half else 'bf16'}, "
                         "22 local(W=512)+4 global, one launch",
@@ -346,8 +348,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="headline decode workload only")
     ap.add_argument("--no-pipeline", action="store_true",
-                    help="skip the 1024 / 256 protocol run through the C++ executor (thousands of small launches: "
-                         "left out of rocprofv3 runs)")
+                    help="skip the legs that call the way an executor does: the 1024 / 256 protocol run through the "
+                         "C++ executor and prefill as one launch per layer (thousands of small launches: left out "
+                         "of rocprofv3 runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for rocprofv3 --pmc counters)")
     args = ap.parse_args()
@@ -411,13 +414,14 @@ def main():
     }
 
     if not args.no_extras:
-        pre = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4))
+        pre = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4),
+                               by_layer=not args.no_pipeline)
         log(f"[bench] prefill C2: {pre['ms_per_step']:.3f} ms/step, {pre['kernel_TFLOPs']:.1f} TFLOP/s kernel")
         result["prefill"] = {
             "workload": pre["workload"], "value": round(pre["TFLOPs"], 2), "unit": "TFLOP/s", "dtype": "bf16",
             "ms_per_step": round(pre["ms_per_step"], 4), "prefill_tokens_per_s": round(pre["tokens_per_s"], 1),
             "single_global_layer_ms": round(pre["single_global_layer_ms"], 4),
-            "layer_by_layer": {
+            "layer_by_layer": None if args.no_pipeline else {
                 "what": "the same 26 layers as 26 launches in turn (how an executor calls it); key ranges of a "
                         "launch this small are cut into parts that a second kernel merges (option "
                         "prefill_key_split, default by rule), *_unsplit: with that switched off",

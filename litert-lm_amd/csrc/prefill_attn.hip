@@ -700,7 +700,23 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
     for (int u = 0; u < units; ++u) b.unit_order[u] = (uint16_t)order[u];
     b.use_order = 1;
   }
-  const long all_items = (long)items * (a.kchunk > 0 ? a.smax : 1);  // (some of them empty when tiles are split)
+  long all_items = items;
+  if (a.kchunk > 0 && a.host_window) {
+    // work items of a key split: the parts that hold at least one key block (the tickets also
+    // number the empty ones, which the drawing thread skips)
+    const int tiles = (a.n + kStretch * pt - 1) / (kStretch * pt);
+    all_items = 0;
+    for (int li = 0; li < a.n_layers; ++li) {
+      const int w = a.host_window[a.layer_begin + li];
+      for (int t = 0; t < tiles; ++t) {
+        const int p0 = a.q_pos0 + t * kStretch * pt;
+        const int last = std::min(p0 + kStretch * pt, a.q_pos0 + a.n) - 1;
+        const int lo = (w > 0 && p0 - w + 1 > 0) ? (p0 - w + 1) / kKeysPerBlock : 0;
+        const int nblk = last / kKeysPerBlock - lo + 1;
+        all_items += (long)((nblk + a.kchunk - 1) / a.kchunk) * a.geom.hkv * (G / hpb);
+      }
+    }
+  }
   int wgs = all_items < cus ? (int)all_items : cus;
   if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
   const dim3 grid(wgs, 1, 1);
