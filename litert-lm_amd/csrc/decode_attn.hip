@@ -296,24 +296,40 @@ __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buff
 // on other XCDs are only guaranteed visible across a kernel boundary; an
 // in-kernel "last arrival merges" needs an L2 write-back and invalidate per
 // workgroup, which measured several times slower than this launch.
-template <int KV, int IO, int D>
+// Grid (query head, sequence, layer). INL and the argument loads in front of the
+// first read of the partials: as in decode_attn_kernel.
+template <int KV, int IO, int D, bool INL>
 __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
   using io_t = typename IoT<IO>::type;
   __shared__ float sm_m[kMaxDecodeSplits], sm_l[kMaxDecodeSplits];
-  const int head = blockIdx.x, item = blockIdx.y, d = threadIdx.x;
-  const int li = item / a.batch, b = item - li * a.batch;
-  const int layer = a.layer_begin + li;
-  const int kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
-  const int window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
+  const int head = blockIdx.x, b = blockIdx.y, li = blockIdx.z, d = threadIdx.x;
+  int batch = a.batch, layer_begin = a.layer_begin, num_splits = a.num_splits, max_kv_len = a.max_kv_len, hq = a.hq;
+  const float* ws_ml = a.ws_ml;
+  const float* ws_acc = a.ws_acc;
+  int kv_len = 0, window = 0;
+  if constexpr (INL) {
+    kv_len = a.inline_lens[b];
+    window = a.inline_window[li];
+  }
+  asm volatile("" : "+s"(batch), "+s"(layer_begin), "+s"(num_splits), "+s"(max_kv_len), "+s"(hq), "+s"(ws_ml),
+               "+s"(ws_acc), "+s"(kv_len), "+s"(window));
+  const int item = li * batch + b;
+  const int layer = layer_begin + li;
+  if constexpr (!INL) {
+    kv_len = a.inline_items ? a.inline_lens[b] : a.kv_lens[b];
+    window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
+    kv_len = __builtin_amdgcn_readfirstlane(kv_len);
+    window = __builtin_amdgcn_readfirstlane(window);
+  }
   int vlo, start;
   decode_visible_range(kv_len, window, &vlo, &start);
-  const int per = decode_partition_tokens(a.max_kv_len, window, a.num_splits);
+  const int per = decode_partition_tokens(max_kv_len, window, num_splits);
   int nparts = (kv_len - start + per - 1) / per;
-  nparts = nparts < a.num_splits ? nparts : a.num_splits;
-  const int64_t slot0 = ((int64_t)item * a.hq + head) * a.num_splits;
+  nparts = nparts < num_splits ? nparts : num_splits;
+  const int64_t slot0 = ((int64_t)item * hq + head) * num_splits;
   // one round trip for all (max, sum) pairs, then the weights come from LDS
   for (int s = d; s < nparts; s += D) {
-    const float2 ml = *reinterpret_cast<const float2*>(a.ws_ml + (slot0 + s) * 2);
+    const float2 ml = *reinterpret_cast<const float2*>(ws_ml + (slot0 + s) * 2);
     sm_m[s] = ml.x;
     sm_l[s] = ml.y;
   }
@@ -322,7 +338,7 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
   for (int s = 0; s < nparts; ++s) M = fmaxf(M, sm_m[s]);
   const float m_use = (M == -INFINITY) ? 0.f : M;
   float A = 0.f, L = 0.f;
-  const float* accp = a.ws_acc + slot0 * D + d;
+  const float* accp = ws_acc + slot0 * D + d;
   int s = 0;
   for (; s + 8 <= nparts; s += 8) {
     float v[8];
@@ -345,7 +361,7 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
     const int seq = a.inline_items ? a.inline_seq[b] : (a.seq_ids ? a.seq_ids[b] : b);
     o *= a.scales[a.geom.scale_offset(layer, seq, 1, head / a.group) + d];
   }
-  reinterpret_cast<io_t*>(a.out)[((int64_t)item * a.hq + head) * D + d] = (io_t)o;
+  reinterpret_cast<io_t*>(a.out)[((int64_t)item * hq + head) * D + d] = (io_t)o;
 }
 
 // INL: lengths, sequence ids and windows travel in the argument block (the host
@@ -492,7 +508,6 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
 
 template <int KV, int IO, int D, int NW, bool INL>
 hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
-  const int items = a.n_layers * a.batch;
   const dim3 grid(a.batch, a.n_layers, a.num_splits * a.geom.hkv);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
@@ -501,7 +516,7 @@ hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, h
   hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || a.num_splits == 1) return err;
-  hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D>), dim3(a.hq, items), dim3(D), 0, stream, a);
+  hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D, INL>), dim3(a.hq, a.batch, a.n_layers), dim3(D), 0, stream, a);
   return hipGetLastError();
 }
 
