@@ -175,6 +175,42 @@ def test_decode_ragged_lengths_and_seq_ids(kv):
         assert err < TOL[kv]
 
 
+def test_decode_more_sequences_and_layers_than_the_argument_block_holds():
+    """Lengths, sequence ids and windows travel in the kernel's argument block for up to 64 sequences
+    and 64 layers; beyond that the kernels read them from device arrays (another kernel variant)."""
+    kv = A.F16
+    # 70 sequences in one layer
+    B = 70
+    rng = np.random.default_rng(70)
+    lens = [int(x) for x in rng.integers(1, 200, size=B)]
+    with make(1, 8, 2, 200, B, kv) as at:
+        kvs = [fill_seq(at, kv, 0, b, gen(700 + b, lens[b], 2, D), gen(800 + b, lens[b], 2, D)) for b in range(B)]
+        q = gen(71, B, 8, D)
+        for ns in (1, 3):
+            err, _ = run_decode(at, kv, q, kvs, lens, num_splits=ns)
+            say(f"70 sequences splits={ns}: rel_err={err:.3e}")
+            assert err < TOL[kv]
+    # 70 layers in one call, windows alternating
+    nl, L = 70, 150
+    windows = [0 if l % 2 == 0 else 20 + l for l in range(nl)]
+    with make(nl, 4, 1, L, 2, kv, layer_window=windows) as at:
+        kd, kr = dev(gen(72, L, 1, D), kv)
+        vd, vr = dev(gen(73, L, 1, D), kv)
+        for layer in range(nl):
+            for b in range(2):
+                at.kv_append(layer, b, 0, kd, vd)
+        qd, qr = dev(gen(74, nl, 2, 4, D), kv)
+        out = torch.empty_like(qd)
+        lens2 = [L, 77]
+        at.decode(0, lens2, qd, out, num_splits=2, n_layers=nl)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        for layer in (0, 1, 33, 68, 69):
+            for b, n in enumerate(lens2):
+                ref = c_oracle.sdpa_f64(qr[layer, b:b + 1], kr, vr, D ** -0.5, q_pos0=n - 1, window=windows[layer], kv_len=n)[0]
+                assert err_of(got[layer, b], ref, kv) < TOL[kv], (layer, b)
+
+
 @pytest.mark.parametrize("kv", [A.F32, A.F16])
 def test_decode_sliding_window_layers(kv):
     windows = [0, 512, 1, 37, 64, 100]
