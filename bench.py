@@ -40,6 +40,10 @@ METRIC = "decode-attn HBM GB/s (% of 8 TB/s) + prefill-attn TFLOP/s, Gemma3n-E2B
 # scaled by what the same counter reads for a plain copy of known size
 # (profiles/bench_default_hbm_traffic.txt): 123,054 KiB x 2.0 fetched + 3,900 KiB x 1.0 written.
 MEASURED_TRAFFIC_BYTES = 256008192
+# The same for the 26-layer bf16 prefill launch: 132,335 KiB x 2.0 fetched past L2 (most of it served by the
+# Infinity Cache: the counter sits between L2 and the memory side) + 53,298 KiB written (the outputs, once);
+# algorithmic: 79,872 KiB read + 53,248 KiB written.
+MEASURED_PREFILL_TRAFFIC_BYTES = (132335 * 2 + 53298) * 1024
 
 
 def log(*a):
@@ -431,7 +435,7 @@ def main():
             "dense_counted_TFLOPs": round(pre["dense_counted_TFLOPs"], 2),
             "roofline": {"kernel": "prefill_attn_kernel<bf16,256>", "bound": "mfma",
                          "achieved": round(pre["kernel_TFLOPs"], 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(pre["frac_of_mfma_peak"], 4), "traffic": None,
+                         "frac": round(pre["frac_of_mfma_peak"], 4), "traffic": MEASURED_PREFILL_TRAFFIC_BYTES,
                          "algorithmic_flops_per_launch": pre["flops"], "avg_kernel_us": round(pre["kernel_ms"] * 1e3, 2)},
         }
         pre16 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), half=True)
