@@ -238,6 +238,11 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      (the only path for fp32 and int8 caches)
  *   "prefill_workgroups" upper bound of the persistent workgroups of the prefill
  *                      kernel, 0 (default) = one per compute unit
+ *   "prefill_rows16"   which of the two prefill kernels runs: 1 the one on 16x16x32 MFMAs
+ *                      (four waves of 32 query positions, 80 KiB of LDS, two workgroups
+ *                      per compute unit), 0 the one on 32x32x16 MFMAs (one workgroup per
+ *                      compute unit), -1 (default): the first when the launch has at least
+ *                      two work items per compute unit, else the second
  *   "prefill_key_split" -1 (default): a prefill launch with fewer work items than
  *                      three quarters of the compute units (a single layer, say) cuts
  *                      the key range of its tiles into up to 8 work items each and

@@ -143,6 +143,7 @@ struct PrefillArgs {
   int32_t kchunk, smax;
   float* ws_acc;
   float* ws_ml;
+  int32_t rows16;  // 1: the kernel on 16x16x32 MFMAs, two workgroups per compute unit; 0: the one on 32x32x16; < 0: by rule
   uint16_t unit_order[128];
 };
 constexpr int kPrefillQueues = 2;                     // ticket queues; workgroup k draws from queue k % 2 first

@@ -75,6 +75,7 @@ struct mi355_attn {
   float* d_pf_ml = nullptr;
   size_t pf_rows = 0;          // rows (of head_dim / of 2 floats) the two hold
   int prefill_key_split = -1;  // < 0 by rule, 0 off, > 0 key blocks per work item
+  int prefill_rows16 = -1;     // which prefill kernel: 1 the one on 16x16x32 MFMAs, 0 the one on 32x32x16, < 0 by rule
   // the step before attention: per-layer constants in HBM and what is switched on
   struct LayerTransform {
     bool set = false, rope = false, norm_q = false, norm_k = false, norm_v = false, q_scaled = false, k_scaled = false;
@@ -327,6 +328,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.softcap = h->cfg.softcap;
     a.max_workgroups = h->prefill_workgroups;
     a.single_p = h->bf16_single_p ? 1 : 0;
+    a.rows16 = h->prefill_rows16;
     a.host_window = h->window.data();
     PrefillSplit split = plan_prefill_split(a, h->prefill_key_split);
     constexpr size_t kSplitRowsMax = (size_t)256 << 10;  // 256 Ki rows = 258 MiB at head_dim 256
@@ -771,6 +773,9 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   } else if (!strcmp(name, "prefill_workgroups")) {
     if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_workgroups = value;
+  } else if (!strcmp(name, "prefill_rows16")) {
+    if (value < -1 || value > 1) return MI355_ATTN_INVALID_ARGUMENT;
+    h->prefill_rows16 = value;
   } else if (!strcmp(name, "prefill_key_split")) {
     if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_key_split = value;

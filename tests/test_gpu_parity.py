@@ -305,12 +305,17 @@ def run_prefill(at, dt, q, kr, vr, q_pos0, window, layer=0, rowwise=False, scale
     return err_of(out.float().cpu().numpy(), ref, dt), out
 
 
+ROWS16 = pytest.mark.parametrize("rows16", [0, 1], ids=["mfma32", "mfma16"])  # the two prefill kernels
+
+
+@ROWS16
 @pytest.mark.parametrize("dt", [A.BF16, A.F16])
 @pytest.mark.parametrize("hq,hkv", [(4, 1), (8, 2), (2, 2), (2, 1), (3, 1)])
-def test_prefill_small_shapes(dt, hq, hkv):
+def test_prefill_small_shapes(dt, hq, hkv, rows16):
     windows = [0, 40, 1, 33]
     L = 400
     with make(len(windows), hq, hkv, L, 1, dt, layer_window=windows) as at:
+        at.set_option("prefill_rows16", rows16)
         k, v = gen(61, L, hkv, D), gen(62, L, hkv, D)
         for layer, w in enumerate(windows):
             kr, vr = fill_seq(at, dt, layer, 0, k, v)
@@ -323,7 +328,8 @@ def test_prefill_small_shapes(dt, hq, hkv):
         say(f"prefill small dt={dt} hq={hq} hkv={hkv}: ok")
 
 
-def test_prefill_bf16_one_operand_per_probability():
+@ROWS16
+def test_prefill_bf16_one_operand_per_probability(rows16):
     # option "prefill_bf16_single_p": P enters the P.V product as one bf16 value. Error beyond the output
     # format's own rounding stays under 2e-3 (max-norm); with the output rounding the L2 figure is
     # 2.0e-3 .. 2.5e-3 (the default, split, path stays under 2e-3, see err_of), bound here at 3e-3.
@@ -331,6 +337,7 @@ def test_prefill_bf16_one_operand_per_probability():
     L, hq, hkv = 1024, 4, 1
     windows = [0, 512, 1]
     with make(len(windows), hq, hkv, L, 1, A.BF16, layer_window=windows) as at:
+        at.set_option("prefill_rows16", rows16)
         at.set_option("prefill_bf16_single_p", 1)
         k, v = gen(161, L, hkv, D), gen(162, L, hkv, D)
         for layer, w in enumerate(windows):
@@ -351,10 +358,12 @@ def test_prefill_bf16_one_operand_per_probability():
                 assert beyond < TOL[A.BF16] and l2 < 3e-3
 
 
-def test_prefill_c2_full_size_local_and_global():
+@ROWS16
+def test_prefill_c2_full_size_local_and_global(rows16):
     # config 2: 1024-token chunk, Hq4/Hkv1, bf16; one local (W=512) and one global layer
     seed = orc.SEED_BASE + 1
     with make(2, 4, 1, 1024, 1, A.BF16, layer_window=[512, 0]) as at:
+        at.set_option("prefill_rows16", rows16)
         for layer, w in ((0, 512), (1, 0)):
             q = gen(seed + layer, 1024, 4, D)
             kr, vr = fill_seq(at, A.BF16, layer, 0, gen(seed + 10 + layer, 1024, 1, D), gen(seed + 20 + layer, 1024, 1, D))
@@ -390,15 +399,17 @@ def test_prefill_chunked_equals_one_shot_and_layers_call():
         assert orc.rel_err(two.float().cpu().numpy(), one.float().cpu().numpy()) < TOL[A.BF16]
 
 
+@ROWS16
 @pytest.mark.parametrize("dt", [A.BF16, A.F16])
 @pytest.mark.parametrize("hq,hkv,kchunk", [(4, 1, 1), (4, 1, 3), (8, 2, 2), (3, 1, 5), (2, 2, 4)])
-def test_prefill_key_split_matches_oracle(dt, hq, hkv, kchunk):
+def test_prefill_key_split_matches_oracle(dt, hq, hkv, kchunk, rows16):
     """Tiles cut into work items of `kchunk` key blocks whose parts a second kernel merges: global and
     windowed layers, ragged ends, a later chunk of a longer context, rows that see no key of a part
     (causal: the early rows of a tile and its last part; window: the late rows and its first part)."""
     windows = [0, 40, 1, 33, 200]
     L = 700
     with make(len(windows), hq, hkv, L, 1, dt, layer_window=windows) as at:
+        at.set_option("prefill_rows16", rows16)
         at.set_option("prefill_key_split", kchunk)
         k, v = gen(261, L, hkv, D), gen(262, L, hkv, D)
         for layer, w in enumerate(windows):
@@ -435,16 +446,19 @@ def test_prefill_key_split_by_rule_softcap_and_limits():
         say(f"key split by rule: rel_err {err:.3e}, unsplit {err0:.3e}")
     # soft cap (the visibility test then follows the cap) and a scale of its own
     with make(1, 4, 2, 300, 1, A.F16, layer_window=[70], scale=0.09, softcap=5.0) as at:
-        at.set_option("prefill_key_split", 2)
         kr, vr = fill_seq(at, A.F16, 0, 0, gen(281, 300, 2, D), gen(282, 300, 2, D))
         qd, qr = dev(gen(283, 250, 4, D), A.F16)
-        out = torch.empty_like(qd)
-        at.prefill(0, 0, 50, 250, qd, out)
-        torch.cuda.synchronize()
         ref = c_oracle.sdpa_f64(qr, kr, vr, 0.09, q_pos0=50, window=70, softcap=5.0, kv_len=300)
-        err = err_of(out.float().cpu().numpy(), ref, A.F16)
-        say(f"key split with soft cap: rel_err {err:.3e}")
-        assert err < TOL[A.F16]
+        for rows16 in (0, 1):
+            for ks in (0, 2):
+                at.set_option("prefill_rows16", rows16)
+                at.set_option("prefill_key_split", ks)
+                out = torch.empty_like(qd)
+                at.prefill(0, 0, 50, 250, qd, out)
+                torch.cuda.synchronize()
+                err = err_of(out.float().cpu().numpy(), ref, A.F16)
+                say(f"soft cap, kernel {rows16}, key split {ks}: rel_err {err:.3e}")
+                assert err < TOL[A.F16]
     # a forced split whose parts would not fit the workspace limit is refused, not shrunk
     with make(1, 8, 2, 8192, 1, A.F16) as at:
         at.set_option("prefill_key_split", 1)
@@ -460,9 +474,10 @@ def test_prefill_key_split_by_rule_softcap_and_limits():
             at.set_option("prefill_key_split", -2)
 
 
+@ROWS16
 @pytest.mark.parametrize("dt", [A.F16, A.BF16])
 @pytest.mark.parametrize("hq,hkv,key_split", [(4, 1, 0), (8, 4, 0), (3, 1, 0), (4, 1, 3), (8, 4, 2)])
-def test_prefill_many_work_items_per_workgroup(dt, hq, hkv, key_split):
+def test_prefill_many_work_items_per_workgroup(dt, hq, hkv, key_split, rows16):
     """Few persistent workgroups walking many work items each (what one launch over 26 layers does on
     the full chip): the hand-over between items -- tickets, rings, query rows, output rows or parts of
     split tiles -- must not depend on how many workgroups share the queue. Short and long items,
@@ -471,6 +486,7 @@ def test_prefill_many_work_items_per_workgroup(dt, hq, hkv, key_split):
     nl, n, pos0 = 5, 333, 160
     windows = [0, 70, 0, 512, 33]
     with make(nl, hq, hkv, pos0 + n, 1, dt, layer_window=windows) as at:
+        at.set_option("prefill_rows16", rows16)
         at.set_option("prefill_key_split", key_split)
         qd, _ = dev(gen(91, nl, n, hq, D), dt)
         for layer in range(nl):
@@ -634,10 +650,12 @@ def test_golden_vectors(path, dt):
                 err = err_of(out.float().cpu().numpy(), want, dt)
                 assert err < TOL[dt], (os.path.basename(path), dt, splits, err)
         else:
-            at.prefill(0, 0, q_pos0, n, qd, out)
-            torch.cuda.synchronize()
-            err = err_of(out.float().cpu().numpy(), want, dt)
-            assert err < TOL[dt], (os.path.basename(path), dt, err)
+            for rows16 in ((0, 1) if dt != A.F32 else (0,)):  # both MFMA kernels
+                at.set_option("prefill_rows16", rows16)
+                at.prefill(0, 0, q_pos0, n, qd, out)
+                torch.cuda.synchronize()
+                err = err_of(out.float().cpu().numpy(), want, dt)
+                assert err < TOL[dt], (os.path.basename(path), dt, rows16, err)
         say(f"golden {os.path.basename(path)} dt={dt}: rel_err={err:.3e}")
 
 
