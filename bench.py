@@ -154,7 +154,8 @@ def prefill_flops(n, hq, window):
     return 4 * hq * D * pairs
 
 
-def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, single_p=False, by_layer=False):
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, single_p=False, by_layer=False,
+                     rows16=-1):
     hq, hkv = 4, 1
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
     stream = torch.cuda.current_stream().cuda_stream
@@ -162,6 +163,7 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, sin
     at = A.Attn(layers, hq, hkv, D, n, 1, dt, dt, layer_window=windows, stream=stream)
     if single_p:
         at.set_option("prefill_bf16_single_p", 1)
+    at.set_option("prefill_rows16", rows16)
     fill_cache(at, torch, layers, [n], hkv, tdt, seed=0xC0FFEE + 1)
     q = torch.randn((layers, n, hq, D), device="cuda:0").to(tdt)
     out = torch.empty_like(q)
@@ -433,7 +435,7 @@ def main():
                 "unsplit_ms": round(pre["layer_by_layer_unsplit_ms"], 4),
                 "single_global_layer_unsplit_ms": round(pre["single_global_layer_unsplit_ms"], 4)},
             "dense_counted_TFLOPs": round(pre["dense_counted_TFLOPs"], 2),
-            "roofline": {"kernel": "prefill_attn_kernel<bf16,256>", "bound": "mfma",
+            "roofline": {"kernel": "prefill_attn16_kernel<bf16,256>", "bound": "mfma",
                          "achieved": round(pre["kernel_TFLOPs"], 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(pre["frac_of_mfma_peak"], 4), "traffic": MEASURED_PREFILL_TRAFFIC_BYTES,
                          "algorithmic_flops_per_launch": pre["flops"], "avg_kernel_us": round(pre["kernel_ms"] * 1e3, 2)},
@@ -444,6 +446,14 @@ def main():
                                   "kernel_TFLOPs": round(pre16["kernel_TFLOPs"], 2),
                                   "frac_of_mfma_peak": round(pre16["frac_of_mfma_peak"], 4),
                                   "avg_kernel_us": round(pre16["kernel_ms"] * 1e3, 2)}
+        pre32 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), rows16=0)
+        log(f"[bench] prefill C2 with the 32x32x16-MFMA kernel: {pre32['ms_per_step']:.3f} ms/step, "
+            f"{pre32['kernel_TFLOPs']:.1f} TFLOP/s kernel")
+        result["prefill_mfma32_kernel"] = {
+            "workload": pre32["workload"] + ", option prefill_rows16=0: the kernel with one workgroup per CU that "
+                                            "small launches use (the default picks the 16x16x32 kernel here)",
+            "value": round(pre32["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre32["kernel_TFLOPs"], 2),
+            "frac_of_mfma_peak": round(pre32["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre32["kernel_ms"] * 1e3, 2)}
         pre1 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), single_p=True)
         log(f"[bench] prefill C2, bf16 with one operand per probability: {pre1['ms_per_step']:.3f} ms/step, "
             f"{pre1['kernel_TFLOPs']:.1f} TFLOP/s kernel")
