@@ -27,6 +27,7 @@
 // (runtime/executor/llm_litert_compiled_model_executor.cc:271) and the
 // [1,1,S,ctx] mask built for it
 // (runtime/executor/litert_compiled_model_executor_utils.cc:332-397).
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <math.h>
 
@@ -948,12 +949,14 @@ __global__ void __launch_bounds__(D) prefill_merge_kernel(const PrefillArgs a, i
 template <int DT, int D, int HPB, bool CAP, bool SPLITP>
 hipError_t launch_variant(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill_lds_bytes<D>();
-  static bool configured = false;  // more than 64 KiB of LDS has to be requested once per kernel
-  if (!configured) {
+  // more than 64 KiB of LDS has to be requested once per kernel (callers on several threads may both
+  // make the request; it is idempotent)
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB, CAP, SPLITP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
   hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB, CAP, SPLITP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
@@ -964,12 +967,12 @@ hipError_t launch_variant(const PrefillArgs& a, dim3 grid, hipStream_t stream, h
 template <int DT, int D, int HPB, bool CAP, bool SPLITP>
 hipError_t launch_variant16(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill16_lds_bytes<D>();
-  static bool configured = false;
-  if (!configured) {
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn16_kernel<DT, D, HPB, CAP, SPLITP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   hipExtLaunchKernelGGL((prefill_attn16_kernel<DT, D, HPB, CAP, SPLITP>), grid, dim3(kWaves16 * 64), kLds, stream, ev0,
                         ev1, 0, a);
@@ -1002,12 +1005,14 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
   const int pt = 4 / hpb;
   const int items = a.n_layers * a.geom.hkv * (G / hpb) * ((a.n + kStretch * pt - 1) / (kStretch * pt));
-  static int cus = 0;  // one persistent workgroup per CU
+  static std::atomic<int> cus_cached{0};  // persistent workgroups are sized by the CU count
+  int cus = cus_cached.load(std::memory_order_relaxed);
   if (cus == 0) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
+    cus_cached.store(cus, std::memory_order_relaxed);
   }
   PrefillArgs b = a;
   b.use_order = 0;
