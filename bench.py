@@ -323,7 +323,7 @@ def pipeline_report(X):
     return r["report"], float(pre.group(1)), float(dec.group(1))
 
 
-def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=12.0):
+def cpu_baseline_c3(layers, ctx, step_bytes, budget_s=24.0):
     """C restatement of the reference CPU op order (fp32, OpenMP) on the same
     30-layer decode sweep, repeated until about `budget_s` seconds are spent."""
     from oracle import c_oracle
@@ -505,7 +505,7 @@ def main():
             "unit": "GB/s",
             "cores": ref_threads,
             "kind": "port",
-            "sample": f"{cpu[ref_threads]['reps']} passes of the same 30-layer decode sweep (fp32 K/V copies, about 6 s), "
+            "sample": f"{cpu[ref_threads]['reps']} passes of the same 30-layer decode sweep (fp32 K/V copies, about 12 s), "
                       "C restatement of the reference CPU op order (oracle/attn_oracle.c, OpenMP); "
                       "4 threads = the reference's CpuConfig default; bytes counted as for the GPU (fp16 sizes)",
             "ms_per_step": round(cpu[ref_threads]["sec_per_step"] * 1e3, 3),
