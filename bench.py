@@ -114,14 +114,14 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
             "single_layer_latency_us": lat * 1e6, "tokens_per_s": 1.0 / sec}
 
 
-def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits):
-    """Single-layer batched decode (configs 4 and 5), rotating over `rotation` layers."""
+def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits, layers=1):
+    """Batched decode (configs 4 and 5): `layers` layers per launch, rotating over `rotation` sets of them."""
     hq, hkv = 8, 2
     B = len(lens)
     stream = torch.cuda.current_stream().cuda_stream
-    at = A.Attn(rotation, hq, hkv, D, 4096, B, kv, A.F16, stream=stream)
+    at = A.Attn(rotation * layers, hq, hkv, D, 4096, B, kv, A.F16, stream=stream)
     g = torch.Generator(device="cuda:0").manual_seed(0xC0FFEE + (3 if kv == A.F16 else 4))
-    for layer in range(rotation):
+    for layer in range(rotation * layers):
         for b, n in enumerate(lens):
             if kv == A.I8:
                 k = torch.randint(-127, 128, (n, hkv, D), generator=g, device="cuda:0", dtype=torch.int8)
@@ -132,17 +132,17 @@ def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits
                 k = torch.randn((n, hkv, D), generator=g, device="cuda:0").half()
                 v = torch.randn((n, hkv, D), generator=g, device="cuda:0").half()
             at.kv_append(layer, b, 0, k, v)
-    q = torch.randn((B, hq, D), device="cuda:0").half()
+    q = torch.randn((layers, B, hq, D), device="cuda:0").half()
     out = torch.empty_like(q)
     clens = A._i32_array(lens)
 
     def step(i):
-        at.decode(i % rotation, clens, q, out, num_splits=splits, batch=B)
+        at.decode((i % rotation) * layers, clens, q, out, num_splits=splits, n_layers=layers, batch=B)
 
     sec = time_steps(torch, step, steps, warmup)
     kms = kernel_ms(torch, at, step, steps, warmup + steps)
     esz = 1 if kv == A.I8 else 2
-    nbytes = sum(lens) * hkv * D * 2 * esz + 2 * B * hq * D * 2 + (B * 2 * hkv * D * 4 if kv == A.I8 else 0)
+    nbytes = layers * (sum(lens) * hkv * D * 2 * esz + 2 * B * hq * D * 2 + (B * 2 * hkv * D * 4 if kv == A.I8 else 0))
     at.close()
     return {"workload": name, "ms_per_step": sec * 1e3, "kernel_ms": kms, "bytes": nbytes,
             "GBps": nbytes / sec / 1e9, "kernel_GBps": nbytes / (kms * 1e-3) / 1e9,
@@ -468,9 +468,16 @@ def main():
         rng = np.random.default_rng(0xC0FFEE + 3)
         lens4 = [int(x) for x in rng.integers(256, 4097, size=64)]
         extras = []
-        for name, kv, lens, rot in (("C4: 64 seqs, L~U[256,4096], fp16, one layer", A.F16, lens4, 4),
-                                    ("C5: 32 seqs x 4096, int8 KV + fp32 scales, one layer", A.I8, [4096] * 32, 6)):
-            r = bench_decode_batch(A, torch, name, kv, lens, max(20, args.steps // 4), max(5, args.warmup // 4), rot, 16)
+        # (the 16-layer launches sweep 2 to 4.5 GB of cache each: nothing of it stays in L2 or the Infinity Cache)
+        for name, kv, lens, rot, nl in (("C4: 64 seqs, L~U[256,4096], fp16, one layer", A.F16, lens4, 4, 1),
+                                        ("C5: 32 seqs x 4096, int8 KV + fp32 scales, one layer", A.I8, [4096] * 32, 6, 1),
+                                        ("C4 x 16 layers in one launch, split count by the library's rule (none)", A.F16, lens4, 1, 16),
+                                        ("C5 x 16 layers in one launch, split count by the library's rule (none)", A.I8, [4096] * 32, 1, 16),
+                                        ("32 seqs x 4096, fp16, 16 layers in one launch, split count by the library's rule (none)", A.F16, [4096] * 32, 1, 16)):
+            # split count: 16 for one layer; the library's own rule (num_splits 0) for the 16-layer launches,
+            # which have a workgroup per wave slot without any split
+            r = bench_decode_batch(A, torch, name, kv, lens, max(20, args.steps // 4), max(5, args.warmup // 4), rot,
+                                   16 if nl == 1 else 0, layers=nl)
             log(f"[bench] {name}: {r['ms_per_step']*1e3:.1f} us/step, kernel {r['kernel_GBps']:.0f} GB/s")
             extras.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()})
         c1 = bench_decode_c1(A, torch, args.steps, args.warmup)

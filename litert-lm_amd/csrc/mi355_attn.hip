@@ -250,8 +250,10 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   HIP_OR_RETURN(hipSetDevice(h->device));
   const int items = n_layers * batch;
   if (num_splits == 0) {
-    // enough workgroups to cover the chip a few times, partitions of >= 64 tokens
-    const int want = (2048 + items * h->cfg.num_kv_heads - 1) / (items * h->cfg.num_kv_heads);
+    // About 1024 workgroups (four waves per CU saturate HBM; measured: 30 layers x 2 KV heads at 4096 tokens
+    // run 8 % faster with 16-18 partitions than with 35, 16 layers x 64 sequences fastest without any split),
+    // partitions of >= 64 tokens.
+    const int want = (1024 + items * h->cfg.num_kv_heads - 1) / (items * h->cfg.num_kv_heads);
     num_splits = std::max(1, std::min({want, (max_len + 63) / 64, 64}));
   }
   DecodeArgs a{};
