@@ -86,9 +86,11 @@ struct DecodeArgs {
   float* ws_ml;              // [items][hq][num_splits][2] partial (max, sum)
   const int32_t* kv_lens;    // [batch] (unused when inline_items != 0)
   const int32_t* seq_ids;    // [batch] or nullptr
-  int32_t inline_items;      // != 0: batch <= kInlineItems and lens / sequence ids travel in the argument block
+  int32_t inline_items;      // != 0: batch <= kInlineItems and lens / sequence ids travel in the argument block,
+                             // in dispatch order (longest sequence first): entry j belongs to batch row inline_row[j]
   int32_t inline_lens[kInlineItems];
   int32_t inline_seq[kInlineItems];
+  int32_t inline_row[kInlineItems];
   const int32_t* layer_window;  // [num_layers] (read only when n_layers > kInlineLayers)
   int32_t inline_window[kInlineLayers];  // windows of layers layer_begin .. layer_begin + n_layers - 1
   CacheGeom geom;
@@ -96,6 +98,7 @@ struct DecodeArgs {
   int32_t layer_begin, n_layers, batch;
   int32_t num_splits;
   int32_t max_kv_len;        // max over kv_lens (host computed), sizes the partitions
+  int32_t min_kv_len;        // min over kv_lens (host computed; only the launch rules look at it)
   float scale;               // softmax scale
   float softcap;
 };

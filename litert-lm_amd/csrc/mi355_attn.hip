@@ -227,10 +227,11 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
                 h->cfg.max_seqs);
   if (num_splits < 0 || num_splits > kMaxSplits)
     return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "num_splits %d outside [0, %d]", num_splits, kMaxSplits);
+  if (batch > 65535) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "batch %d exceeds the launch grid (65535)", batch);
   if (!decode_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim))
     return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "decode: unsupported kv/io dtype pair %d/%d",
                 h->cfg.kv_dtype, h->cfg.io_dtype);
-  int max_len = 0;
+  int max_len = 0, min_len = INT32_MAX;
   for (int b = 0; b < batch; ++b) {
     const int seq = seq_ids ? seq_ids[b] : b;
     if (seq < 0 || seq >= h->cfg.max_seqs)
@@ -246,6 +247,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
                     "kv_lens[%d]=%d but only %d rows of layer %d, sequence %d were appended", b, len,
                     h->filled[(size_t)l * h->cfg.max_seqs + seq], l, seq);
     max_len = std::max(max_len, len);
+    min_len = std::min(min_len, len);
   }
   HIP_OR_RETURN(hipSetDevice(h->device));
   const int items = n_layers * batch;
@@ -267,9 +269,15 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
   if (batch <= kInlineItems) {
     a.inline_items = 1;
-    for (int b = 0; b < batch; ++b) {
-      a.inline_lens[b] = kv_lens[b];
-      a.inline_seq[b] = seq_ids ? seq_ids[b] : b;
+    // dispatch order: longest sequence first (rows keep their places in q and out)
+    int order[kInlineItems];
+    for (int b = 0; b < batch; ++b) order[b] = b;
+    std::stable_sort(order, order + batch, [&](int x, int y) { return kv_lens[x] > kv_lens[y]; });
+    for (int j = 0; j < batch; ++j) {
+      const int b = order[j];
+      a.inline_lens[j] = kv_lens[b];
+      a.inline_seq[j] = seq_ids ? seq_ids[b] : b;
+      a.inline_row[j] = b;
     }
   } else if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, error_msg)) {
     return rc;
@@ -281,6 +289,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   a.batch = batch;
   a.num_splits = num_splits;
   a.max_kv_len = max_len;
+  a.min_kv_len = min_len;
   fill_inline_windows(h, &a);
   HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream,
                               h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr));

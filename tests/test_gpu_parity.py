@@ -211,6 +211,52 @@ def test_decode_more_sequences_and_layers_than_the_argument_block_holds():
                 assert err_of(got[layer, b], ref, kv) < TOL[kv], (layer, b)
 
 
+@pytest.mark.parametrize("kv", [A.F16, A.I8])
+def test_decode_many_layers_of_a_ragged_batch_in_one_launch(kv):
+    """A serving step: 8 layers x 64 sequences of unequal lengths in one call. The library picks the
+    split count (none: the launch has 1024 workgroups without), dispatches the longest sequences first
+    (rows of q and out keep the caller's order) and, lengths being unequal, runs four waves per
+    workgroup; sequence ids are a permutation, so slot, row and dispatch order all differ."""
+    nl, B, hq, hkv, L = 8, 64, 8, 2, 320
+    rng = np.random.default_rng(88)
+    lens = [int(x) for x in rng.integers(1, L + 1, size=B)]
+    lens[5], lens[40] = L, 1
+    seq_ids = [int(x) for x in rng.permutation(B)]
+    windows = [0, 100, 0, 0, 33, 0, 0, 0]
+    with make(nl, hq, hkv, L, B, kv, layer_window=windows) as at:
+        rows = {}
+        k0, v0 = gen(881, L, hkv, D), gen(882, L, hkv, D)
+        for layer in range(nl):
+            for b in range(B):  # contents differ per (layer, sequence): a rolled copy of one tensor
+                shift = 7 * layer + 3 * b
+                k = np.roll(k0, shift, axis=0)[:lens[b]]
+                v = np.roll(v0, shift, axis=0)[:lens[b]]
+                if kv == A.I8:
+                    kq, ks = orc.quantize_kv_int8(k)
+                    vq, vs = orc.quantize_kv_int8(v)
+                    at.kv_append(layer, seq_ids[b], 0, torch.from_numpy(kq).to(DEV), torch.from_numpy(vq).to(DEV))
+                    at.kv_set_scales(layer, seq_ids[b], torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
+                    rows[(layer, b)] = (orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs))
+                else:
+                    rows[(layer, b)] = fill_seq(at, kv, layer, seq_ids[b], k, v)
+        qd, qr = dev(gen(883, nl, B, hq, D), A.F16 if kv == A.I8 else kv)
+        out = torch.full_like(qd, float("nan"))
+        at.decode(0, lens, qd, out, seq_ids=seq_ids, num_splits=0, n_layers=nl)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        worst = 0.0
+        for layer in range(nl):
+            for b in (0, 5, 17, 40, 63, int(np.argmax(lens)), int(np.argmin(lens))):
+                kr_, vr_ = rows[(layer, b)]
+                n = lens[b]
+                ref = c_oracle.sdpa_f64(qr[layer, b:b + 1], kr_, vr_, D ** -0.5, q_pos0=n - 1, window=windows[layer], kv_len=n)[0]
+                e = err_of(got[layer, b], ref, kv)
+                worst = max(worst, e)
+                assert e < TOL[kv], (layer, b, n, e)
+        say(f"8 layers x 64 ragged sequences kv={kv}: worst rel_err={worst:.3e}")
+
+
 @pytest.mark.parametrize("kv", [A.F32, A.F16])
 def test_decode_sliding_window_layers(kv):
     windows = [0, 512, 1, 37, 64, 100]
