@@ -84,8 +84,9 @@ struct DecodeArgs {
   const float* scales;       // int8 cache only
   float* ws_acc;             // [items][hq][num_splits][D] partial accumulators
   float* ws_ml;              // [items][hq][num_splits][2] partial (max, sum)
-  const int32_t* kv_lens;    // [batch] (unused when inline_items != 0)
+  const int32_t* kv_lens;    // [batch] in dispatch order (unused when inline_items != 0)
   const int32_t* seq_ids;    // [batch] or nullptr
+  const int32_t* rows;       // [batch] row in q / out of dispatch slot j (batches beyond kInlineItems), or nullptr
   int32_t inline_items;      // != 0: batch <= kInlineItems and lens / sequence ids travel in the argument block,
                              // in dispatch order (longest sequence first): entry j belongs to batch row inline_row[j]
   int32_t inline_lens[kInlineItems];

@@ -316,6 +316,8 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
                "+s"(ws_acc), "+s"(kv_len), "+s"(window), "+s"(b));
   if constexpr (!INL) {
     if (a.inline_items) b = a.inline_row[j];
+    else if (a.rows) b = a.rows[j];
+    b = __builtin_amdgcn_readfirstlane(b);
   }
   const int item = li * batch + b;
   const int layer = layer_begin + li;
@@ -406,15 +408,16 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   asm volatile("" : "+s"(hkv), "+s"(batch), "+s"(layer_begin), "+s"(max_seqs), "+s"(num_splits), "+s"(max_kv_len),
                "+s"(plane_bytes), "+s"(cache), "+s"(seq), "+s"(kv_len), "+s"(window), "+s"(b));
   const int split = blockIdx.z / hkv, kvh = blockIdx.z - split * hkv;
-  const int item = li * batch + b;
   const int layer = layer_begin + li;
   if constexpr (!INL) {
     seq = a.inline_items ? a.inline_seq[j] : (a.seq_ids ? a.seq_ids[j] : j);
     kv_len = a.inline_items ? a.inline_lens[j] : a.kv_lens[j];
     if (a.inline_items) b = a.inline_row[j];
+    else if (a.rows) b = a.rows[j];
     window = a.n_layers <= kInlineLayers ? a.inline_window[li] : a.layer_window[layer];
   }
   b = __builtin_amdgcn_readfirstlane(b);
+  const int item = li * batch + b;  // row of q, out and the partials
   seq = __builtin_amdgcn_readfirstlane(seq);
   kv_len = __builtin_amdgcn_readfirstlane(kv_len);
   window = __builtin_amdgcn_readfirstlane(window);

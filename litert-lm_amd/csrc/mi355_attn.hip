@@ -172,23 +172,30 @@ int ensure_workspace(mi355_attn* h, size_t slots, char** error_msg) {
   return 0;
 }
 
-// Uploads kv_lens (and seq_ids) through a ring of pinned slots so that calls
-// can be queued back to back without waiting for earlier uploads.
+// Uploads lengths, cache slots and rows in dispatch order (longest sequence
+// first) through a ring of pinned slots so that calls can be queued back to
+// back without waiting for earlier uploads.
 int upload_items(mi355_attn* h, const int32_t* seq_ids, const int32_t* kv_lens, int batch,
-                 const int32_t** d_lens, const int32_t** d_seq, char** error_msg) {
+                 const int32_t** d_lens, const int32_t** d_seq, const int32_t** d_rows, char** error_msg) {
   const int slot = h->ring_next;
   h->ring_next = (slot + 1) % kRingSlots;
   if (h->ring_used[slot]) HIP_OR_RETURN(hipEventSynchronize(h->ring_ev[slot]));
   int32_t* hs = h->h_ring + (size_t)slot * h->ring_slot_ints;
   int32_t* ds = h->d_ring + (size_t)slot * h->ring_slot_ints;
-  memcpy(hs, kv_lens, sizeof(int32_t) * batch);
-  if (seq_ids) memcpy(hs + batch, seq_ids, sizeof(int32_t) * batch);
-  const size_t bytes = sizeof(int32_t) * batch * (seq_ids ? 2 : 1);
+  int32_t* order = hs + 2 * (size_t)batch;
+  for (int b = 0; b < batch; ++b) order[b] = b;
+  std::stable_sort(order, order + batch, [&](int x, int y) { return kv_lens[x] > kv_lens[y]; });
+  for (int j = 0; j < batch; ++j) {
+    hs[j] = kv_lens[order[j]];
+    hs[batch + j] = seq_ids ? seq_ids[order[j]] : order[j];
+  }
+  const size_t bytes = sizeof(int32_t) * batch * 3;
   HIP_OR_RETURN(hipMemcpyAsync(ds, hs, bytes, hipMemcpyHostToDevice, h->stream));
   HIP_OR_RETURN(hipEventRecord(h->ring_ev[slot], h->stream));
   h->ring_used[slot] = true;
   *d_lens = ds;
-  *d_seq = seq_ids ? ds + batch : nullptr;
+  *d_seq = ds + batch;
+  *d_rows = ds + 2 * (size_t)batch;
   return 0;
 }
 
@@ -279,7 +286,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
       a.inline_seq[j] = seq_ids ? seq_ids[b] : b;
       a.inline_row[j] = b;
     }
-  } else if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, error_msg)) {
+  } else if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, &a.rows, error_msg)) {
     return rc;
   }
   a.q = dq;
@@ -509,7 +516,7 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
     return bail(MI355_ATTN_INTERNAL, "layer transform clear", e);
   if ((e = hipMemsetAsync(h->d_sched, 0, sizeof(int32_t) * kPrefillSchedInts, h->stream)) != hipSuccess)
     return bail(MI355_ATTN_INTERNAL, "prefill queue clear", e);
-  h->ring_slot_ints = 2 * c->max_seqs;
+  h->ring_slot_ints = 3 * c->max_seqs;
   if ((e = hipHostMalloc(&h->h_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)
     return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "pinned ring", e);
   if ((e = hipMalloc(&h->d_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)

@@ -183,11 +183,12 @@ def test_decode_more_sequences_and_layers_than_the_argument_block_holds():
     B = 70
     rng = np.random.default_rng(70)
     lens = [int(x) for x in rng.integers(1, 200, size=B)]
+    slots = [int(x) for x in rng.permutation(B)]  # row b lives in cache slot slots[b]; dispatch order is a third order
     with make(1, 8, 2, 200, B, kv) as at:
-        kvs = [fill_seq(at, kv, 0, b, gen(700 + b, lens[b], 2, D), gen(800 + b, lens[b], 2, D)) for b in range(B)]
+        kvs = [fill_seq(at, kv, 0, slots[b], gen(700 + b, lens[b], 2, D), gen(800 + b, lens[b], 2, D)) for b in range(B)]
         q = gen(71, B, 8, D)
         for ns in (1, 3):
-            err, _ = run_decode(at, kv, q, kvs, lens, num_splits=ns)
+            err, _ = run_decode(at, kv, q, kvs, lens, num_splits=ns, seq_ids=slots)
             say(f"70 sequences splits={ns}: rel_err={err:.3e}")
             assert err < TOL[kv]
     # 70 layers in one call, windows alternating
@@ -201,7 +202,7 @@ def test_decode_more_sequences_and_layers_than_the_argument_block_holds():
                 at.kv_append(layer, b, 0, kd, vd)
         qd, qr = dev(gen(74, nl, 2, 4, D), kv)
         out = torch.empty_like(qd)
-        lens2 = [L, 77]
+        lens2 = [77, L]  # (the longer sequence second: dispatch order differs from row order)
         at.decode(0, lens2, qd, out, num_splits=2, n_layers=nl)
         torch.cuda.synchronize()
         got = out.float().cpu().numpy()
