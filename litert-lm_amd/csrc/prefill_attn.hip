@@ -825,17 +825,38 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
         const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
         m_run[u] = m_new;
         float lsum = 0.f;
+        if constexpr (SPLITP) {
+          // bf16 high and low parts, two probabilities at a time: one packed conversion gives both high
+          // parts, whose float values are the two halves of that word (a shift and a mask), one more
+          // the low parts (a conversion per element would cost a third more instructions here)
+          static_assert(DT == kBF16, "the two-part probabilities are a bf16 device");
+          typedef float f2 __attribute__((ext_vector_type(2)));
+          typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+          u4 hi_w, lo_w;
 #pragma unroll
-        for (int T = 0; T < 2; ++T)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float pv = fast_exp2(fmaf(sc[u][T][e], c, neg_m));
-            const elem_t hi = (elem_t)pv;
-            p_hi[u][4 * T + e] = hi;
-            if constexpr (SPLITP) p_lo[u][4 * T + e] = (elem_t)(pv - (float)hi);
-            else if constexpr (DT == kBF16) pv = (float)hi;  // the row sum over the rounded values
-            lsum += pv;
+          for (int w = 0; w < 4; ++w) {
+            const int T = w >> 1, e = 2 * (w & 1);
+            const f2 pv = {fast_exp2(fmaf(sc[u][T][e], c, neg_m)), fast_exp2(fmaf(sc[u][T][e + 1], c, neg_m))};
+            const unsigned hw = bit_cast<unsigned>(__builtin_convertvector(pv, b2));
+            const f2 rest = {pv[0] - __uint_as_float(hw << 16), pv[1] - __uint_as_float(hw & 0xffff0000u)};
+            hi_w[w] = hw;
+            lo_w[w] = bit_cast<unsigned>(__builtin_convertvector(rest, b2));
+            lsum += pv[0] + pv[1];
           }
+          p_hi[u] = bit_cast<vec8>(hi_w);
+          p_lo[u] = bit_cast<vec8>(lo_w);
+        } else {
+#pragma unroll
+          for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float pv = fast_exp2(fmaf(sc[u][T][e], c, neg_m));
+              const elem_t hi = (elem_t)pv;
+              p_hi[u][4 * T + e] = hi;
+              if constexpr (DT == kBF16) pv = (float)hi;  // the row sum over the rounded values
+              lsum += pv;
+            }
+        }
         l_run[u] = l_run[u] * alpha + lsum;
         if (__any(alpha != 1.f)) {
 #pragma unroll
