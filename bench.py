@@ -40,10 +40,10 @@ METRIC = "decode-attn HBM GB/s (% of 8 TB/s) + prefill-attn TFLOP/s, Gemma3n-E2B
 # scaled by what the same counter reads for a plain copy of known size
 # (profiles/bench_default_hbm_traffic.txt): 123,054 KiB x 2.0 fetched + 3,900 KiB x 1.0 written.
 MEASURED_TRAFFIC_BYTES = 256008192
-# The same for the 26-layer bf16 prefill launch: 167,214 KiB x 2.0 fetched past L2 (most of it served by the
-# Infinity Cache: the counter sits between L2 and the memory side) + 63,546 KiB written (the outputs once and
+# The same for the 26-layer bf16 prefill launch: 167,410 KiB x 2.0 fetched past L2 (most of it served by the
+# Infinity Cache: the counter sits between L2 and the memory side) + 64,058 KiB written (the outputs once and
 # about 10 MiB of register spills); algorithmic: 79,872 KiB read + 53,248 KiB written.
-MEASURED_PREFILL_TRAFFIC_BYTES = (167214 * 2 + 63546) * 1024
+MEASURED_PREFILL_TRAFFIC_BYTES = (167410 * 2 + 64058) * 1024
 
 
 def log(*a):
