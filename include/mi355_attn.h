@@ -242,7 +242,11 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      (four waves of 32 query positions, 80 KiB of LDS, two workgroups
  *                      per compute unit), 0 the one on 32x32x16 MFMAs (one workgroup per
  *                      compute unit), -1 (default): the first when the launch has at least
- *                      two work items per compute unit, else the second
+ *                      two work items per compute unit, else the second; 2: an
+ *                      experimental third (eight waves per workgroup, two groups of four
+ *                      half an iteration apart; launches it does not take, i.e. key splits
+ *                      and head groups that are no multiple of 4, run kernel 1), never
+ *                      chosen by the rule
  *   "prefill_key_split" -1 (default): a prefill launch with fewer work items than
  *                      three quarters of the compute units (a single layer, say) cuts
  *                      the key range of its tiles into up to 8 work items each and

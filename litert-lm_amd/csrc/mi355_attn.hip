@@ -792,7 +792,7 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
     if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_workgroups = value;
   } else if (!strcmp(name, "prefill_rows16")) {
-    if (value < -1 || value > 1) return MI355_ATTN_INVALID_ARGUMENT;
+    if (value < -1 || value > 2) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_rows16 = value;
   } else if (!strcmp(name, "prefill_key_split")) {
     if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;

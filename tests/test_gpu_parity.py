@@ -352,7 +352,7 @@ def run_prefill(at, dt, q, kr, vr, q_pos0, window, layer=0, rowwise=False, scale
     return err_of(out.float().cpu().numpy(), ref, dt), out
 
 
-ROWS16 = pytest.mark.parametrize("rows16", [0, 1], ids=["mfma32", "mfma16"])  # the two prefill kernels
+ROWS16 = pytest.mark.parametrize("rows16", [0, 1, 2], ids=["mfma32", "mfma16", "mfma16x2"])  # the prefill kernels (2 falls back to 1 for shapes it does not take)
 
 
 @ROWS16
@@ -697,7 +697,7 @@ def test_golden_vectors(path, dt):
                 err = err_of(out.float().cpu().numpy(), want, dt)
                 assert err < TOL[dt], (os.path.basename(path), dt, splits, err)
         else:
-            for rows16 in ((0, 1) if dt != A.F32 else (0,)):  # both MFMA kernels
+            for rows16 in ((0, 1, 2) if dt != A.F32 else (0,)):  # every MFMA kernel
                 at.set_option("prefill_rows16", rows16)
                 at.prefill(0, 0, q_pos0, n, qd, out)
                 torch.cuda.synchronize()
