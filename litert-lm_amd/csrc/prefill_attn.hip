@@ -959,6 +959,8 @@ __global__ void __launch_bounds__(kWaves16x2 * 64) prefill_attn16x2_kernel(const
   constexpr int NL = D / 16;  // 16-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;
   constexpr int kXfers = 16 / kWaves16x2;
+  constexpr int kAheadX2 = 3;  // operand reads in flight (one fewer than the four-wave kernel: a register reloaded inside
+                               // the loop would wait for every transfer under way)
   auto mfma = [](vec8 x, vec8 y, f4 z) {
     if constexpr (DT == kF16) return mfma16_f16(x, y, z);
     else return mfma16_bf16(x, y, z);
@@ -1119,18 +1121,18 @@ __global__ void __launch_bounds__(kWaves16x2 * 64) prefill_attn16x2_kernel(const
 #pragma unroll
         for (int T = 0; T < 2; ++T) sc[u][T] = f4{0.f, 0.f, 0.f, 0.f};
       {
-        // operand reads run kOpAhead steps ahead of the MFMAs that use them (an LDS read takes longer
+        // operand reads run kAheadX2 steps ahead of the MFMAs that use them (an LDS read takes longer
         // than the two MFMAs of a step)
         auto k_at = [&](int step) { return *reinterpret_cast<const vec8*>(kb + (step & 1) * (16 * D * 2) + (step >> 1) * 1024); };
-        vec8 kop[kOpAhead];
+        vec8 kop[kAheadX2];
 #pragma unroll
-        for (int st = 0; st < kOpAhead; ++st) kop[st] = k_at(st);
+        for (int st = 0; st < kAheadX2; ++st) kop[st] = k_at(st);
 #pragma unroll
         for (int st = 0; st < 2 * NJ; ++st) {
           const int j = st >> 1, T = st & 1;
 #pragma unroll
-          for (int u = 0; u < kSub16; ++u) sc[u][T] = mfma(kop[st % kOpAhead], q[u][j], sc[u][T]);
-          if (st + kOpAhead < 2 * NJ) kop[st % kOpAhead] = k_at(st + kOpAhead);
+          for (int u = 0; u < kSub16; ++u) sc[u][T] = mfma(kop[st % kAheadX2], q[u][j], sc[u][T]);
+          if (st + kAheadX2 < 2 * NJ) kop[st % kAheadX2] = k_at(st + kAheadX2);
         }
       }
       // score sc[u][T][e]: key key0 + 16 T + 4 g + e against query my_pos0 + 16 u + n
@@ -1204,17 +1206,17 @@ __global__ void __launch_bounds__(kWaves16x2 * 64) prefill_attn16x2_kernel(const
     auto pv_half = [&](int i) {
       const uint8_t* vb = sm_v + (i % kStagesX2) * kBlockBytes + lane * 16;
       {
-        vec8 vop[kOpAhead];
+        vec8 vop[kAheadX2];
 #pragma unroll
-        for (int st = 0; st < kOpAhead; ++st) vop[st] = *reinterpret_cast<const vec8*>(vb + st * 1024);
+        for (int st = 0; st < kAheadX2; ++st) vop[st] = *reinterpret_cast<const vec8*>(vb + st * 1024);
 #pragma unroll
         for (int db = 0; db < NL; ++db) {
 #pragma unroll
           for (int u = 0; u < kSub16; ++u) {
-            acc[u][db] = mfma(vop[db % kOpAhead], p_hi[u], acc[u][db]);
-            if constexpr (SPLITP) acc[u][db] = mfma(vop[db % kOpAhead], p_lo[u], acc[u][db]);
+            acc[u][db] = mfma(vop[db % kAheadX2], p_hi[u], acc[u][db]);
+            if constexpr (SPLITP) acc[u][db] = mfma(vop[db % kAheadX2], p_lo[u], acc[u][db]);
           }
-          if (db + kOpAhead < NL) vop[db % kOpAhead] = *reinterpret_cast<const vec8*>(vb + (db + kOpAhead) * 1024);
+          if (db + kAheadX2 < NL) vop[db % kAheadX2] = *reinterpret_cast<const vec8*>(vb + (db + kAheadX2) * 1024);
         }
       }
     };
