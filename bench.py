@@ -454,14 +454,6 @@ def main():
                                             "small launches use (the default picks the 16x16x32 kernel here)",
             "value": round(pre32["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre32["kernel_TFLOPs"], 2),
             "frac_of_mfma_peak": round(pre32["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre32["kernel_ms"] * 1e3, 2)}
-        pre2 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), rows16=2)
-        log(f"[bench] prefill C2 with the eight-wave kernel: {pre2['ms_per_step']:.3f} ms/step, "
-            f"{pre2['kernel_TFLOPs']:.1f} TFLOP/s kernel")
-        result["prefill_mfma16x2_kernel"] = {
-            "workload": pre2["workload"] + ", option prefill_rows16=2: eight waves per workgroup, two groups of four "
-                                           "half an iteration apart (experimental, never chosen by the rule)",
-            "value": round(pre2["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre2["kernel_TFLOPs"], 2),
-            "frac_of_mfma_peak": round(pre2["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre2["kernel_ms"] * 1e3, 2)}
         pre1 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), single_p=True)
         log(f"[bench] prefill C2, bf16 with one operand per probability: {pre1['ms_per_step']:.3f} ms/step, "
             f"{pre1['kernel_TFLOPs']:.1f} TFLOP/s kernel")

@@ -103,6 +103,10 @@ void mi355_attn_destroy(mi355_attn* handle);
  * (llm_litert_npu_compiled_model_executor.cc:105-110,1294-1333).
  * For an int8 cache k and v hold int8 values; set the scales with
  * mi355_attn_kv_set_scales.
+ * Rows count as appended (for the checks of prefill and decode) while they extend
+ * the unbroken prefix [0, rows appended so far) of their layer and sequence: rows
+ * written behind a gap are stored but not counted, so the unwritten rows of the
+ * gap (or, after mi355_attn_reset, a previous sequence's) are never attended to.
  */
 int mi355_attn_kv_append(mi355_attn* handle, int32_t layer, int32_t seq, int32_t pos, int32_t n,
                          const void* k, const void* v, char** error_msg);
@@ -242,11 +246,7 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      (four waves of 32 query positions, 80 KiB of LDS, two workgroups
  *                      per compute unit), 0 the one on 32x32x16 MFMAs (one workgroup per
  *                      compute unit), -1 (default): the first when the launch has at least
- *                      two work items per compute unit, else the second; 2: an
- *                      experimental third (eight waves per workgroup, two groups of four
- *                      half an iteration apart; launches it does not take, i.e. key splits
- *                      and head groups that are no multiple of 4, run kernel 1), never
- *                      chosen by the rule
+ *                      two work items per compute unit, else the second
  *   "prefill_key_split" -1 (default): a prefill launch with fewer work items than
  *                      three quarters of the compute units (a single layer, say) cuts
  *                      the key range of its tiles into up to 8 work items each and

@@ -199,6 +199,14 @@ int upload_items(mi355_attn* h, const int32_t* seq_ids, const int32_t* kv_lens, 
   return 0;
 }
 
+// Rows count as appended only while they extend the unbroken prefix [0, filled) of their
+// (layer, sequence): rows written behind a gap are stored, but attention never takes the unwritten
+// (or, after a reset, stale) rows of the gap for appended ones.
+void note_rows_written(mi355_attn* h, int layer, int seq, int pos, int n) {
+  int32_t& f = h->filled[(size_t)layer * h->cfg.max_seqs + seq];
+  if (pos <= f) f = std::max(f, pos + n);
+}
+
 int check_layers(const mi355_attn* h, int layer_begin, int n_layers, char** error_msg) {
   if (layer_begin < 0 || n_layers < 1 || layer_begin + n_layers > h->cfg.num_layers)
     return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "layers [%d, %d) outside [0, %d)", layer_begin,
@@ -377,6 +385,9 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     if (!decode_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim))
       return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "prefill: unsupported kv/io dtype pair %d/%d",
                   h->cfg.kv_dtype, h->cfg.io_dtype);
+    if (n > 65535)
+      return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
+                  "row-wise prefill (fp32 / int8 cache): %d rows exceed the launch grid (65535); call in chunks", n);
     if (h->d_items_cap < (size_t)n) {
       HIP_OR_RETURN(hipStreamSynchronize(h->stream));
       if (h->d_items) HIP_OR_RETURN(hipFree(h->d_items));
@@ -472,6 +483,13 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
   h->geom.cap = (int32_t)round_up64(c->max_tokens, kTokenAlign);
   h->geom.esize = dtype_size(c->kv_dtype);
   h->geom.plane_bytes = (int64_t)h->geom.cap * c->head_dim * h->geom.esize;
+  // the kernels address a plane through a 32-bit buffer descriptor and 32-bit block offsets
+  if (h->geom.plane_bytes > (int64_t)INT32_MAX) {
+    const long long pb = (long long)h->geom.plane_bytes;
+    delete h;
+    return fail(error_msg, MI355_ATTN_UNIMPLEMENTED, "max_tokens %d: one plane would hold %lld bytes (limit 2 GiB - 1)",
+                c->max_tokens, pb);
+  }
   h->cache_bytes = (uint64_t)h->geom.plane_bytes * 2 * c->num_kv_heads * c->max_seqs * c->num_layers;
 
   auto bail = [&](int code, const char* what, hipError_t e) {
@@ -584,8 +602,7 @@ int mi355_attn_kv_append(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos,
   a.v = const_cast<void*>(dv);
   HIP_OR_RETURN(launch_kv_append(a, h->stream));
   if (h->cfg.host_io) HIP_OR_RETURN(hipStreamSynchronize(h->stream));
-  int32_t& f = h->filled[(size_t)layer * h->cfg.max_seqs + seq];
-  f = std::max(f, pos + n);
+  note_rows_written(h, layer, seq, pos, n);
   return MI355_ATTN_OK;
 }
 
@@ -691,8 +708,7 @@ int mi355_attn_pre_attention(mi355_attn* h, int32_t layer, int32_t seq, int32_t 
   HIP_OR_RETURN(launch_pre_attention(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, h->timing ? h->ev0 : nullptr,
                                      h->timing ? h->ev1 : nullptr));
   h->timed = h->timing;
-  int32_t& f = h->filled[(size_t)layer * h->cfg.max_seqs + seq];
-  f = std::max(f, pos + n);
+  note_rows_written(h, layer, seq, pos, n);
   return stage_out_end(h, 1, q_out, q_bytes, error_msg);
 }
 
@@ -792,7 +808,7 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
     if (value < 0) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_workgroups = value;
   } else if (!strcmp(name, "prefill_rows16")) {
-    if (value < -1 || value > 2) return MI355_ATTN_INVALID_ARGUMENT;
+    if (value < -1 || value > 1) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_rows16 = value;
   } else if (!strcmp(name, "prefill_key_split")) {
     if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;

@@ -80,6 +80,8 @@ constexpr int prefill_lds_bytes() { return 2 * kStages * 64 * D + kWaves * kStre
 
 // s_waitcnt immediates (gfx9 encoding: vmcnt[3:0], expcnt[6:4], lgkmcnt[11:8],
 // vmcnt[15:14]) that wait on vector-memory operations only.
+// "all but the n most recent vector-memory operations of this wave have completed" (n <= 63)
+constexpr int wait_vm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 constexpr int kWaitVm0 = 0x0F70;  // all of this wave's transfers have landed
 constexpr int kWaitVm4 = 0x0F74;  // all but the 4 most recent ones
 constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
@@ -767,7 +769,7 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
     const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
     // K(0) has to be there for everybody (the query loads, issued last, may still be under way;
     // the compiler waits for those where it needs them)
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (kSub16 * NJ));
+    __builtin_amdgcn_s_waitcnt(wait_vm(kSub16 * NJ));
     lds_barrier();
 
     for (int i = 0; i < nblk; ++i) {
@@ -864,7 +866,7 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
         }
       }
       // this wave's share of V(i) (and of K(i + 1)) has landed; K(i + 2) may be under way
-      if (more_k) __builtin_amdgcn_s_waitcnt(0x0F70 | kXfers);
+      if (more_k) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       lds_barrier();
       if (more_v) fetch(vplane, sm_v, kVStages16, i + 1);
@@ -908,367 +910,6 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
         constexpr int kRowStride = 2 * D + 16;
         static_assert(kWaves16 * kRows16 * kRowStride <= kKStages16 * kBlockBytes - 16, "patches below the ticket");
         uint8_t* const patch = sm_k + wave * (kRows16 * kRowStride);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-#pragma unroll
-        for (int db = 0; db < NL; ++db) {
-          elem_t o[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (elem_t)(acc[u][db][e] * inv);
-          *reinterpret_cast<u2*>(patch + n * kRowStride + (16 * db + 4 * g) * 2) = *reinterpret_cast<const u2*>(o);
-        }
-        // (the patch is private to the wave and LDS operations of a wave stay in order: no barrier)
-        const int row_base = my_pos0 + kRows16 * u - a.q_pos0;
-        const int chunk = lane & 31, hh = lane >> 5;
-#pragma unroll
-        for (int jj = 0; jj < kRows16 / 2; ++jj) {
-          const int r = 2 * jj + hh;
-          const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStride + chunk * 16);
-          if (row_base + r < a.n) {
-            elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row_base + r) * a.hq + head) * D;
-            *reinterpret_cast<u4*>(orow + chunk * 8) = w;
-          }
-        }
-      }
-    }
-  }  // next work item
-
-  if (tid == 0) {
-    const int done = atomicAdd(a.sched + kPrefillQueues, 1);
-    if (done == (int)gridDim.x - 1)
-      for (int i = 0; i < kPrefillSchedInts; ++i) atomicExch(a.sched + i, 0);
-  }
-}
-
-// The same arithmetic with both waves of a SIMD in one workgroup: eight waves, two groups of four (one
-// head each) on the first and second 32 positions of a 64-position tile, half an iteration apart (see
-// the ring protocol inside). One workgroup per CU; launches without key split and with four heads per
-// KV head block only.
-constexpr int kWaves16x2 = 8;
-constexpr int kStagesX2 = 3;
-template <int D>
-constexpr int prefill16x2_lds_bytes() { return 2 * kStagesX2 * 64 * D + 16; }  // two rings of three blocks + the ticket
-
-template <int DT, int D, int HPB, bool CAP, bool SPLITP>
-__global__ void __launch_bounds__(kWaves16x2 * 64) prefill_attn16x2_kernel(const PrefillArgs a) {
-  using E = El<DT>;
-  using elem_t = typename E::type;
-  using vec8 = typename E::vec8;
-  static_assert(HPB == 4, "four heads per group of waves");
-  constexpr int kTile = 2 * kStretch;  // positions of a work item: 32 per group of four waves
-  constexpr int NJ = D / 32;  // 32-channel steps of the QK^T product
-  constexpr int NL = D / 16;  // 16-channel tiles of O^T
-  constexpr int kBlockBytes = 64 * D;
-  constexpr int kXfers = 16 / kWaves16x2;
-  constexpr int kAheadX2 = 3;  // operand reads in flight (one fewer than the four-wave kernel: a register reloaded inside
-                               // the loop would wait for every transfer under way)
-  auto mfma = [](vec8 x, vec8 y, f4 z) {
-    if constexpr (DT == kF16) return mfma16_f16(x, y, z);
-    else return mfma16_bf16(x, y, z);
-  };
-
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* const sm_k = smem;
-  uint8_t* const sm_v = smem + kStagesX2 * kBlockBytes;
-  volatile int* const sm_ticket = reinterpret_cast<volatile int*>(smem + 2 * kStagesX2 * kBlockBytes);
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n = lane & 15, g = lane >> 4;
-  const int grp = wave >> 2, hw = wave & 3;  // group of waves (first / second 32 positions of the tile), head in the block
-  const int hblocks = a.group / HPB;
-  const int per_layer = a.geom.hkv * hblocks;
-  const int units = a.n_layers * per_layer;
-  const int tiles = (a.n + kTile - 1) / kTile;
-  const int home = blockIdx.x & (kPrefillQueues - 1);
-  int tried = 0;
-  bool first_draw = true;
-  constexpr int smax = 1;  // (launched without key split only)
-  const float softcap = a.softcap;
-  const float c = CAP ? 1.f : a.scale * kLog2e;
-  const int pos_end = a.q_pos0 + a.n;
-
-  struct Item { int li, kvh, hb, tile, part, layer, window, wg_pos0, kb_lo, nblk_tile; };
-  auto item_of = [&](int qx, int ticket) {
-    Item it;
-    const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
-    const int per_tile = qcnt * smax;
-    const int ti = ticket / per_tile, r2 = ticket - ti * per_tile;
-    it.part = r2 / qcnt;
-    const int slot = qx + kPrefillQueues * (r2 - it.part * qcnt);
-    const int u = a.use_order ? a.unit_order[slot] : slot;
-    it.li = u / per_layer;
-    const int rem = u - it.li * per_layer;
-    it.kvh = rem / hblocks;
-    it.hb = rem - it.kvh * hblocks;
-    it.tile = tiles - 1 - ti;
-    it.layer = a.layer_begin + it.li;
-    it.window = a.layer_window[it.layer];
-    it.wg_pos0 = a.q_pos0 + it.tile * kTile;
-    const int last_pos = min(it.wg_pos0 + kTile, pos_end) - 1;
-    it.kb_lo = 0;
-    if (it.window > 0 && it.wg_pos0 - it.window + 1 > 0) it.kb_lo = (it.wg_pos0 - it.window + 1) / kKeysPerBlock;
-    it.nblk_tile = last_pos / kKeysPerBlock - it.kb_lo + 1;
-    return it;
-  };
-
-  for (;;) {
-    if (tid == 0) {
-      int x = 0, t = -1;
-      while (tried < kPrefillQueues) {
-        x = (home + tried) & (kPrefillQueues - 1);
-        const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;
-        if (cnt > 0) {
-          const int home_wgs = ((int)gridDim.x - x + kPrefillQueues - 1) / kPrefillQueues;
-          if (first_draw && tried == 0) t = (int)blockIdx.x / kPrefillQueues;
-          else t = atomicAdd(a.sched + x, 1) + home_wgs;
-          first_draw = false;
-          if (t < cnt * tiles * smax) {
-            break;
-          }
-          t = -1;
-        }
-        ++tried;
-      }
-      sm_ticket[0] = x;
-      sm_ticket[1] = t;
-    }
-    lds_barrier();  // also: every wave is done with the rings of the previous item
-    const int qx = __builtin_amdgcn_readfirstlane(sm_ticket[0]);
-    const int ticket = __builtin_amdgcn_readfirstlane(sm_ticket[1]);
-    if (ticket < 0) break;
-    const Item it = item_of(qx, ticket);
-    const int li = it.li, kvh = it.kvh, layer = it.layer, window = it.window;
-    const int head = kvh * a.group + it.hb * HPB + hw;
-    const int my_pos0 = it.wg_pos0 + grp * kStretch;  // first of the wave's 32 positions
-    const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
-    const uint8_t* vplane = kplane + a.geom.plane_bytes;
-    const int kb_lo = it.kb_lo;
-    const int nblk = it.nblk_tile;
-
-    auto fetch = [&](const uint8_t* plane, uint8_t* ring, int stages, int i) {
-#pragma unroll
-      for (int t = 0; t < kXfers; ++t) {
-        const int off = (wave + kWaves16x2 * t) * 1024;
-        const uint8_t* src = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16 + off;
-        uint8_t* dst = ring + (i % stages) * kBlockBytes + off;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-      }
-    };
-    // Ring protocol. A block takes two half-steps with a barrier after each: group 0 computes the scores
-    // and probabilities of block i in half-step 2 i and its P.V in 2 i + 1, group 1 one half-step later,
-    // so that in every half-step the MFMAs of one group's P.V run against the softmax arithmetic of the
-    // other on the SIMDs they share. K(i) is read in half-steps 2 i and 2 i + 1, V(i) in 2 i + 1 and
-    // 2 i + 2; three stages each: K(i + 2) is asked for at the top of half-step 2 i (its stage held
-    // K(i - 1), last read in 2 i - 1), V(i + 2) at the top of 2 i + 1 (V(i - 1), last read in 2 i). Every
-    // wave asks in the order K0 V0 K1 V1 K2 V2 ... and, before a barrier, waits for its share of what
-    // group 0 reads next, leaving only the requests made after that one outstanding.
-    fetch(kplane, sm_k, kStagesX2, 0);
-    fetch(vplane, sm_v, kStagesX2, 0);
-    if (nblk > 1) {
-      fetch(kplane, sm_k, kStagesX2, 1);
-      fetch(vplane, sm_v, kStagesX2, 1);
-    }
-
-    // Q^T operands: lane (n, g) holds, for sub-tile u and step j, channels 32 j + 8 g .. + 7 of query my_pos0 + 16 u + n
-    vec8 q[kSub16][NJ];
-#pragma unroll
-    for (int u = 0; u < kSub16; ++u) {
-      const int row = min(my_pos0 + kRows16 * u + n - a.q_pos0, a.n - 1);  // rows past the end repeat the last one; never stored
-      const elem_t* qrow = reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + row) * a.hq + head) * D;
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) q[u][j] = *reinterpret_cast<const vec8*>(qrow + 32 * j + 8 * g);
-    }
-    f4 acc[kSub16][NL];
-#pragma unroll
-    for (int u = 0; u < kSub16; ++u)
-#pragma unroll
-      for (int i = 0; i < NL; ++i) acc[u][i] = f4{0.f, 0.f, 0.f, 0.f};
-    float m_run[kSub16], l_run[kSub16];
-#pragma unroll
-    for (int u = 0; u < kSub16; ++u) { m_run[u] = -INFINITY; l_run[u] = 0.f; }
-    const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
-    const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // the first blocks (and the queries) are there
-    lds_barrier();
-
-    vec8 p_hi[kSub16], p_lo[kSub16];  // probabilities of a block, from its scores half-step to its P.V half-step
-    // top of half-step h: every wave asks for its share of K(h / 2 + 2) (h even) or V(h / 2 + 2) (h odd)
-    auto top_half = [&](int h) {
-      const int i2 = (h >> 1) + 2;
-      if (i2 < nblk) {
-        if (h & 1) fetch(vplane, sm_v, kStagesX2, i2);
-        else fetch(kplane, sm_k, kStagesX2, i2);
-      }
-    };
-    // end of half-step h: what group 0 reads in the next one has to be there: K(i + 1) after an odd
-    // half-step (requests made after it: V(i + 1), K(i + 2), V(i + 2)), V(i) after an even one (K(i + 1),
-    // V(i + 1), K(i + 2)); requests beyond the last block do not exist
-    auto end_half = [&](int h) {
-      const int i = h >> 1;
-      const int later = (h & 1) ? (i + 1 < nblk ? 1 : 0) + (i + 2 < nblk ? 2 : 0) : (i + 1 < nblk ? 2 : 0) + (i + 2 < nblk ? 1 : 0);
-      if (later == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * kXfers));
-      else if (later == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kXfers));
-      else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | kXfers);
-      else __builtin_amdgcn_s_waitcnt(0x0F70);
-      lds_barrier();
-    };
-    auto scores_half = [&](int i) {
-      const uint8_t* kb = sm_k + (i % kStagesX2) * kBlockBytes + lane * 16;
-      f4 sc[kSub16][2];
-#pragma unroll
-      for (int u = 0; u < kSub16; ++u)
-#pragma unroll
-        for (int T = 0; T < 2; ++T) sc[u][T] = f4{0.f, 0.f, 0.f, 0.f};
-      {
-        // operand reads run kAheadX2 steps ahead of the MFMAs that use them (an LDS read takes longer
-        // than the two MFMAs of a step)
-        auto k_at = [&](int step) { return *reinterpret_cast<const vec8*>(kb + (step & 1) * (16 * D * 2) + (step >> 1) * 1024); };
-        vec8 kop[kAheadX2];
-#pragma unroll
-        for (int st = 0; st < kAheadX2; ++st) kop[st] = k_at(st);
-#pragma unroll
-        for (int st = 0; st < 2 * NJ; ++st) {
-          const int j = st >> 1, T = st & 1;
-#pragma unroll
-          for (int u = 0; u < kSub16; ++u) sc[u][T] = mfma(kop[st % kAheadX2], q[u][j], sc[u][T]);
-          if (st + kAheadX2 < 2 * NJ) kop[st % kAheadX2] = k_at(st + kAheadX2);
-        }
-      }
-      // score sc[u][T][e]: key key0 + 16 T + 4 g + e against query my_pos0 + 16 u + n
-      const int key0 = (kb_lo + i) * kKeysPerBlock;
-      const bool all_vis = key0 + kKeysPerBlock - 1 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim;
-#pragma unroll
-      for (int u = 0; u < kSub16; ++u) {
-        const int my_pos = my_pos0 + kRows16 * u + n;
-        float bm = -INFINITY;
-#pragma unroll
-        for (int T = 0; T < 2; ++T)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float x = sc[u][T][e];
-            if constexpr (CAP) x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
-            if (!all_vis) x = (unsigned)(my_pos - (key0 + 16 * T + 4 * g + e)) < wlim ? x : -INFINITY;
-            sc[u][T][e] = x;
-            bm = fmaxf(bm, x);
-          }
-        bm *= c;
-        // The four lanes of a query compare notes only when one of them has seen a score that
-        // exceeds the reference by more than the slack: rare after the first blocks.
-        if (__any(bm > m_run[u] + kRescaleSlack)) {
-          bm = wave_xor_max(bm, 16);
-          bm = wave_xor_max(bm, 32);
-        }
-        const float m_new = bm > m_run[u] + kRescaleSlack ? bm : m_run[u];
-        const float alpha = (m_run[u] == -INFINITY) ? 1.f : fast_exp2(m_run[u] - m_new);
-        const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
-        m_run[u] = m_new;
-        float lsum = 0.f;
-        if constexpr (SPLITP) {
-          // bf16 high and low parts, two probabilities at a time: one packed conversion gives both high
-          // parts, whose float values are the two halves of that word (a shift and a mask), one more
-          // the low parts (a conversion per element would cost a third more instructions here)
-          static_assert(DT == kBF16, "the two-part probabilities are a bf16 device");
-          typedef float f2 __attribute__((ext_vector_type(2)));
-          typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-          u4 hi_w, lo_w;
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            const int T = w >> 1, e = 2 * (w & 1);
-            const f2 pv = {fast_exp2(fmaf(sc[u][T][e], c, neg_m)), fast_exp2(fmaf(sc[u][T][e + 1], c, neg_m))};
-            const unsigned hw = bit_cast<unsigned>(__builtin_convertvector(pv, b2));
-            const f2 rest = {pv[0] - __uint_as_float(hw << 16), pv[1] - __uint_as_float(hw & 0xffff0000u)};
-            hi_w[w] = hw;
-            lo_w[w] = bit_cast<unsigned>(__builtin_convertvector(rest, b2));
-            lsum += pv[0] + pv[1];
-          }
-          p_hi[u] = bit_cast<vec8>(hi_w);
-          p_lo[u] = bit_cast<vec8>(lo_w);
-        } else {
-#pragma unroll
-          for (int T = 0; T < 2; ++T)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float pv = fast_exp2(fmaf(sc[u][T][e], c, neg_m));
-              const elem_t hi = (elem_t)pv;
-              p_hi[u][4 * T + e] = hi;
-              if constexpr (DT == kBF16) pv = (float)hi;  // the row sum over the rounded values
-              lsum += pv;
-            }
-        }
-        l_run[u] = l_run[u] * alpha + lsum;
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-          for (int db = 0; db < NL; ++db) acc[u][db] *= alpha;
-        }
-      }
-    };
-    auto pv_half = [&](int i) {
-      const uint8_t* vb = sm_v + (i % kStagesX2) * kBlockBytes + lane * 16;
-      {
-        vec8 vop[kAheadX2];
-#pragma unroll
-        for (int st = 0; st < kAheadX2; ++st) vop[st] = *reinterpret_cast<const vec8*>(vb + st * 1024);
-#pragma unroll
-        for (int db = 0; db < NL; ++db) {
-#pragma unroll
-          for (int u = 0; u < kSub16; ++u) {
-            acc[u][db] = mfma(vop[db % kAheadX2], p_hi[u], acc[u][db]);
-            if constexpr (SPLITP) acc[u][db] = mfma(vop[db % kAheadX2], p_lo[u], acc[u][db]);
-          }
-          if (db + kAheadX2 < NL) vop[db % kAheadX2] = *reinterpret_cast<const vec8*>(vb + (db + kAheadX2) * 1024);
-        }
-      }
-    };
-    // 2 nblk + 1 half-steps for either group (the barrier counts must agree): group 0 idles in the last
-    // one, group 1 in the first
-    if (grp == 0) {
-      for (int i = 0; i < nblk; ++i) {
-        top_half(2 * i);
-        scores_half(i);
-        end_half(2 * i);
-        top_half(2 * i + 1);
-        pv_half(i);
-        end_half(2 * i + 1);
-      }
-      top_half(2 * nblk);
-      end_half(2 * nblk);
-    } else {
-      top_half(0);
-      end_half(0);
-      for (int i = 0; i < nblk; ++i) {
-        top_half(2 * i + 1);
-        scores_half(i);
-        end_half(2 * i + 1);
-        top_half(2 * i + 2);
-        pv_half(i);
-        end_half(2 * i + 2);
-      }
-    }
-
-    constexpr bool split_tile = false;
-    // ---- store: lane (n, g) holds channels 16 db + 4 g .. + 3 of query my_pos0 + 16 u + n
-#pragma unroll
-    for (int u = 0; u < kSub16; ++u) {
-      float l_tot = wave_xor_add(l_run[u], 16);
-      l_tot = wave_xor_add(l_tot, 32);
-      const int row = my_pos0 + kRows16 * u + n - a.q_pos0;
-      if (row < a.n) {
-        if (split_tile) {
-          const int64_t slot = (((int64_t)li * a.n + row) * a.hq + head) * smax + it.part;
-          float* prow = a.ws_acc + slot * D + 4 * g;
-#pragma unroll
-          for (int db = 0; db < NL; ++db) *reinterpret_cast<f4*>(prow + 16 * db) = acc[u][db];
-          if (g == 0) *reinterpret_cast<float2*>(a.ws_ml + slot * 2) = float2{m_run[u], l_tot};
-        }
-      }
-      if (!split_tile) {
-        // Whole rows through LDS (the K ring is idle: every wave has passed the last barrier of the
-        // loop; each wave has a patch of its own, 16 rows padded to 528 bytes, below the ticket), then
-        // two 512-byte rows per store instruction.
-        constexpr int kRowStride = 2 * D + 16;
-        static_assert(kWaves16x2 * kRows16 * kRowStride <= 2 * kStagesX2 * kBlockBytes, "patches inside the rings");
-        uint8_t* const patch = smem + wave * (kRows16 * kRowStride);
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
 #pragma unroll
         for (int db = 0; db < NL; ++db) {
@@ -1361,34 +1002,8 @@ hipError_t launch_variant16(const PrefillArgs& a, dim3 grid, hipStream_t stream,
   return hipGetLastError();
 }
 
-template <int DT, int D, bool CAP, bool SPLITP>
-hipError_t launch_variant16x2(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
-  constexpr int kLds = prefill16x2_lds_bytes<D>();
-  static std::atomic<bool> configured{false};
-  if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn16x2_kernel<DT, D, 4, CAP, SPLITP>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return e;
-    configured.store(true, std::memory_order_release);
-  }
-  hipExtLaunchKernelGGL((prefill_attn16x2_kernel<DT, D, 4, CAP, SPLITP>), grid, dim3(kWaves16x2 * 64), kLds, stream, ev0,
-                        ev1, 0, a);
-  return hipGetLastError();
-}
-
 template <int DT, int D, int HPB>
 hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
-  if constexpr (HPB == 4) {
-    if (a.rows16 == 2) {
-      if constexpr (DT == kBF16) {
-        if (!a.single_p)
-          return a.softcap > 0.f ? launch_variant16x2<DT, D, true, true>(a, grid, stream, ev0, ev1)
-                                 : launch_variant16x2<DT, D, false, true>(a, grid, stream, ev0, ev1);
-      }
-      return a.softcap > 0.f ? launch_variant16x2<DT, D, true, false>(a, grid, stream, ev0, ev1)
-                             : launch_variant16x2<DT, D, false, false>(a, grid, stream, ev0, ev1);
-    }
-  }
   if (a.rows16) {
     if constexpr (DT == kBF16) {
       if (!a.single_p)
@@ -1469,8 +1084,6 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
   // per CU) when there are at least two work items per CU, else the one on 32x32x16 MFMAs, whose
   // single workgroup per CU gets through an item in half the time.
   b.rows16 = a.rows16 < 0 ? (all_items >= 2L * cus ? 1 : 0) : a.rows16;
-  if (b.rows16 == 2 && (hpb != 4 || a.kchunk > 0)) b.rows16 = 1;  // the eight-wave kernel: four heads per block, whole tiles
-  if (b.rows16 == 2) all_items = (long)units * ((a.n + 2 * kStretch - 1) / (2 * kStretch));
   const int slots = b.rows16 == 1 ? 2 * cus : cus;
   int wgs = all_items < slots ? (int)all_items : slots;
   if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;

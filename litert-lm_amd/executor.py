@@ -103,7 +103,7 @@ class HipLlmExecutor:
     """HipLlmExecutor over the synthetic decoder layers (test scaffolding)."""
 
     def __init__(self, num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens, runner_lengths=(1024,),
-                 layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=True,
+                 layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=False,
                  softcap=0.0, pre_attention=False):
         self._win = _arr(layer_window) if layer_window is not None else None
         self._runners = _arr(runner_lengths)

@@ -27,9 +27,11 @@ struct HipExecutorOptions {
   std::vector<int> prefill_runner_lengths = {1024};
   // The reference loop never runs for a one-id chunk, so a token left pending
   // by an earlier call is overwritten and lost
-  // (llm_litert_compiled_model_executor.cc:187,244). true: execute it first
-  // (this executor's default); false: reproduce the reference.
-  bool execute_pending_on_single_id_chunk = true;
+  // (llm_litert_compiled_model_executor.cc:187,244). false (default): the
+  // reference behaviour, step counts and positions included; true: execute the
+  // pending token first (opt-in fix: GetCurrentStep then reads one higher than
+  // the reference's after such a call).
+  bool execute_pending_on_single_id_chunk = false;
 };
 
 // One forward pass as the executor issued it (kept for tests and debugging).

@@ -99,6 +99,13 @@ KeyValue ReadKeyValue(Wire& w, uint64_t table) {
 Status ReadFileRange(const std::string& path, uint64_t begin, uint64_t end, std::string* out) {
   std::ifstream in(path, std::ios::binary);
   if (!in.is_open()) return InternalError("Could not open file: " + path);
+  // offsets come from the file's own header: they are checked against the file before anything is sized by them
+  in.seekg(0, std::ios::end);
+  const std::streamoff file_size = in.tellg();
+  if (file_size < 0) return InternalError("Could not size file: " + path);
+  if (end < begin || end > static_cast<uint64_t>(file_size))
+    return InvalidArgumentError("Section range [" + std::to_string(begin) + ", " + std::to_string(end) +
+                                ") lies outside the file (" + std::to_string(file_size) + " bytes).");
   in.seekg(static_cast<std::streamoff>(begin));
   out->resize(end - begin);
   in.read(out->data(), static_cast<std::streamsize>(out->size()));

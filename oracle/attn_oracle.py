@@ -355,6 +355,14 @@ def half_ulp_bf16(x) -> np.ndarray:
     return np.where(x > 0, np.ldexp(1.0, ex - 9), 0.0)
 
 
+def round_bf16(x) -> np.ndarray:
+    """x rounded to the nearest bfloat16 (ties to even), returned as float64."""
+    f = np.ascontiguousarray(np.asarray(x, dtype=np.float32))
+    u = f.view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
 def rel_err_beyond_bf16_rounding(a, b) -> float:
     """Norm-wise relative error after discounting, element by element, the
     half-ulp that storing the result as bfloat16 must cost. A bfloat16 output

@@ -17,7 +17,7 @@ X = load_package().executor
 INVALID_ARGUMENT, OUT_OF_RANGE, INTERNAL = 3, 11, 13
 
 
-def make(runners=(1024,), max_tokens=4096, fix=True, **kw):
+def make(runners=(1024,), max_tokens=4096, fix=False, **kw):
     return X.HipLlmExecutor(2, 4, 1, 16, max_tokens, runner_lengths=runners, recording_backend=True,
                             execute_pending_on_single_id_chunk=fix, **kw)
 
@@ -71,6 +71,9 @@ def test_benchmark_shape_1024_ids():
 
 
 def test_single_id_chunk_quirk_and_fix():
+    with X.HipLlmExecutor(2, 4, 1, 16, 64, runner_lengths=(4,), recording_backend=True) as dflt:
+        dflt.prefill([1, 2]); dflt.prefill([3])  # the default is the reference's behaviour
+        assert dflt.runs() == [("prefill", [1], [0]), ("prefill", [], [])] and dflt.current_step() == 2
     with make(runners=(4,), fix=False) as ref:  # reference behaviour: the pending token is dropped
         ref.prefill([1, 2]); ref.prefill([3])
         assert ref.runs() == [("prefill", [1], [0]), ("prefill", [], [])] and ref.current_step() == 2

@@ -31,6 +31,9 @@ def say(*a):
     print(*a, flush=True)
 
 
+BF16_PLAIN = []  # plain norm-wise error of every bf16 comparison of this session (summary test at the end)
+
+
 def err_of(got, ref, dt):
     """The figure held against TOL[dt]. fp32 / fp16 / int8-KV (fp16 output):
     max|a-b| / max|ref|. bf16 output: the same after discounting the half-ulp of
@@ -39,7 +42,14 @@ def err_of(got, ref, dt):
     if dt == A.BF16:
         l2 = orc.l2_rel_err(got, ref)
         assert l2 < TOL[dt], f"bf16 L2-relative error {l2:.3e}"
-        return orc.rel_err_beyond_bf16_rounding(got, ref)
+        beyond = orc.rel_err_beyond_bf16_rounding(got, ref)
+        # the plain norm-wise figure, for the record: it includes the rounding of the bf16 output itself
+        # (up to 2^-8 = 3.9e-3 of an element by format), which no kernel can remove
+        plain = orc.rel_err(got, ref)
+        BF16_PLAIN.append(plain)
+        say(f"    bf16: plain max|a-b|/max|ref| {plain:.3e} (bf16 rounding of the exact result alone: "
+            f"{orc.rel_err(orc.round_bf16(ref), ref):.3e}), beyond output rounding {beyond:.3e}, L2 {l2:.3e}")
+        return beyond
     return orc.rel_err(got, ref)
 
 
@@ -352,7 +362,7 @@ def run_prefill(at, dt, q, kr, vr, q_pos0, window, layer=0, rowwise=False, scale
     return err_of(out.float().cpu().numpy(), ref, dt), out
 
 
-ROWS16 = pytest.mark.parametrize("rows16", [0, 1, 2], ids=["mfma32", "mfma16", "mfma16x2"])  # the prefill kernels (2 falls back to 1 for shapes it does not take)
+ROWS16 = pytest.mark.parametrize("rows16", [0, 1], ids=["mfma32", "mfma16"])  # the two prefill kernels
 
 
 @ROWS16
@@ -417,6 +427,36 @@ def test_prefill_c2_full_size_local_and_global(rows16):
             err, _ = run_prefill(at, A.BF16, q, kr, vr, 0, w, layer=layer)
             say(f"C2 bf16 layer window={w}: rel_err={err:.3e}")
             assert err < TOL[A.BF16]
+
+
+@pytest.mark.parametrize("dt", [A.BF16, A.F16])
+def test_prefill_c2_benched_launch_every_layer(dt):
+    """The launch bench.py times: 26 layers x 1024 tokens, Hq4/Hkv1, windows 512 except every sixth layer
+    (global), all layers in ONE call, kernel and work distribution by the library's own rule. Every
+    layer is compared with the float64 oracle."""
+    layers, n, hq, hkv = 26, 1024, 4, 1
+    windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
+    seed = orc.SEED_BASE + 1
+    with make(layers, hq, hkv, n, 1, dt, layer_window=windows) as at:
+        krs, vrs = [], []
+        for layer in range(layers):
+            kr, vr = fill_seq(at, dt, layer, 0, gen(seed + 100 + layer, n, hkv, D), gen(seed + 200 + layer, n, hkv, D))
+            krs.append(kr)
+            vrs.append(vr)
+        qd, qr = dev(gen(seed + 300, layers, n, hq, D), dt)
+        out = torch.empty_like(qd)
+        for rep in range(2):  # twice: the second launch finds the queue counters as the first left them
+            out.zero_()
+            at.prefill(0, 0, 0, n, qd, out, n_layers=layers)
+            torch.cuda.synchronize()
+            got = out.float().cpu().numpy()
+            worst = 0.0
+            for layer, w in enumerate(windows):
+                ref = c_oracle.sdpa_f64(qr[layer], krs[layer], vrs[layer], D ** -0.5, window=w)
+                err = err_of(got[layer], ref, dt)
+                worst = max(worst, err)
+                assert err < TOL[dt], (dt, rep, layer, w, err)
+            say(f"C2 benched launch dt={dt} pass {rep}: worst layer rel_err {worst:.3e}")
 
 
 def test_prefill_chunked_equals_one_shot_and_layers_call():
@@ -622,11 +662,10 @@ def test_c4_batched_ragged_full_size():
 
 
 def test_c5_int8_full_size_properties():
-    # 32 sequences x 4096 int8; oracle on 4 of them, linearity in V on all
+    # 32 sequences x 4096 int8: every sequence against the oracle, then linearity in the V scales
     B, L = 32, 4096
     with make(1, 8, 2, L, B, A.I8) as at:
         rng = np.random.default_rng(orc.SEED_BASE + 4)
-        check = {0, 7, 19, 31}
         kvs = {}
         for b in range(B):
             k = rng.standard_normal((L, 2, D)).astype(np.float32)
@@ -635,19 +674,20 @@ def test_c5_int8_full_size_properties():
             vq, vs = orc.quantize_kv_int8(v)
             at.kv_append(0, b, 0, torch.from_numpy(kq).to(DEV), torch.from_numpy(vq).to(DEV))
             at.kv_set_scales(0, b, torch.from_numpy(ks).to(DEV), torch.from_numpy(vs).to(DEV))
-            if b in check:
-                kvs[b] = (orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs))
+            kvs[b] = (orc.dequantize_kv_int8(kq, ks), orc.dequantize_kv_int8(vq, vs))
         q = gen(orc.SEED_BASE + 40, B, 8, D)
         qd, qr = dev(q, A.F16)
         out = torch.empty_like(qd)
         at.decode(0, [L] * B, qd, out, num_splits=8)
         torch.cuda.synchronize()
         got = out.float().cpu().numpy()
-        for b in sorted(check):
+        worst = 0.0
+        for b in range(B):
             ref = c_oracle.sdpa_f64(qr[b:b + 1], kvs[b][0], kvs[b][1], D ** -0.5, q_pos0=L - 1)[0]
             err = orc.rel_err(got[b], ref)
-            say(f"C5 full seq {b}: rel_err={err:.3e}")
-            assert err < TOL[A.I8]
+            worst = max(worst, err)
+            assert err < TOL[A.I8], (b, err)
+        say(f"C5 full, all {B} sequences: worst rel_err={worst:.3e}")
         assert np.isfinite(got).all()
         # size-independent property on all 32 sequences: doubling every V scale doubles the output
         for b in range(B):
@@ -697,7 +737,7 @@ def test_golden_vectors(path, dt):
                 err = err_of(out.float().cpu().numpy(), want, dt)
                 assert err < TOL[dt], (os.path.basename(path), dt, splits, err)
         else:
-            for rows16 in ((0, 1, 2) if dt != A.F32 else (0,)):  # every MFMA kernel
+            for rows16 in ((0, 1) if dt != A.F32 else (0,)):  # both MFMA kernels
                 at.set_option("prefill_rows16", rows16)
                 at.prefill(0, 0, q_pos0, n, qd, out)
                 torch.cuda.synchronize()
@@ -763,3 +803,14 @@ def test_host_io_mode():
         dec = np.zeros((1, 4, D), np.float32)
         at.decode(0, [L], q[L - 1:L].copy(), dec, num_splits=2)
         assert orc.rel_err(dec[0], ref[L - 1]) < TOL[A.F32]
+
+
+def test_zz_bf16_plain_error_summary():
+    """Range of the plain norm-wise error max|a-b| / max|ref| over every bf16 comparison of this session
+    (the figure the 2e-3 bound is stated in; for a bf16 output it is dominated by the rounding of the
+    output format itself, which is why err_of also reports the part beyond that rounding)."""
+    if not BF16_PLAIN:
+        pytest.skip("no bf16 comparison ran in this session")
+    say(f"bf16 plain norm-wise error over {len(BF16_PLAIN)} comparisons: min {min(BF16_PLAIN):.3e}, "
+        f"median {float(np.median(BF16_PLAIN)):.3e}, max {max(BF16_PLAIN):.3e}")
+    assert max(BF16_PLAIN) < 2.0 ** -8 + 2e-3  # output rounding (at most 2^-8 of max|ref|) + the stated bound
