@@ -103,9 +103,11 @@ Status ReadFileRange(const std::string& path, uint64_t begin, uint64_t end, std:
   in.seekg(0, std::ios::end);
   const std::streamoff file_size = in.tellg();
   if (file_size < 0) return InternalError("Could not size file: " + path);
-  if (end < begin || end > static_cast<uint64_t>(file_size))
-    return InvalidArgumentError("Section range [" + std::to_string(begin) + ", " + std::to_string(end) +
-                                ") lies outside the file (" + std::to_string(file_size) + " bytes).");
+  if (end < begin)
+    return InvalidArgumentError("Section range [" + std::to_string(begin) + ", " + std::to_string(end) + ") is reversed.");
+  // (a file that ends before the section does: the status of a short read, without sizing anything by the header)
+  if (end > static_cast<uint64_t>(file_size))
+    return InternalError("Could not read " + std::to_string(end - begin) + " bytes from stream.");
   in.seekg(static_cast<std::streamoff>(begin));
   out->resize(end - begin);
   in.read(out->data(), static_cast<std::streamsize>(out->size()));

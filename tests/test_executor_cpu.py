@@ -125,8 +125,8 @@ def test_error_paths():
         with pytest.raises(X.ExecutorError) as e:
             ex.decode()
         assert e.value.code == INVALID_ARGUMENT
-        ex.prefill(list(range(9)))  # 8 executed + 1 pending
-        ex.decode(); ex.decode()    # positions 8, 9
+        ex.prefill(list(range(8)))  # 7 executed + 1 pending
+        ex.decode(); ex.decode(); ex.decode()  # positions 7, 8, 9
         with pytest.raises(X.ExecutorError) as e:
             ex.decode()             # position 10 does not exist
         assert e.value.code == OUT_OF_RANGE

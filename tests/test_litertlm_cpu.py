@@ -239,6 +239,11 @@ def test_hf_tokenizer_round_trip_and_damage(tmp_path):
     with pytest.raises(X.ExecutorError) as e:
         X.litertlm_section(path, 0, X.SECTION_BINARY)
     assert e.value.code == INTERNAL
+    wild = [section(None, 4096, 1 << 62, X.SECTION_BINARY)]               # an end offset far past the file: a status, no allocation
+    path = write(tmp_path, "wild.litertlm", container([], wild, [(4096, b"x" * 10)]))
+    with pytest.raises(X.ExecutorError) as e:
+        X.litertlm_section(path, 0, X.SECTION_BINARY)
+    assert e.value.code == INTERNAL
 
 
 # ------------------------------------------------------------------ damaged preambles and headers
