@@ -154,15 +154,13 @@ def prefill_flops(n, hq, window):
     return 4 * hq * D * pairs
 
 
-def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, single_p=False, by_layer=False,
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_layer=False,
                      rows16=-1):
     hq, hkv = 4, 1
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
     stream = torch.cuda.current_stream().cuda_stream
     dt, tdt = (A.F16, torch.float16) if half else (A.BF16, torch.bfloat16)
     at = A.Attn(layers, hq, hkv, D, n, 1, dt, dt, layer_window=windows, stream=stream)
-    if single_p:
-        at.set_option("prefill_bf16_single_p", 1)
     at.set_option("prefill_rows16", rows16)
     fill_cache(at, torch, layers, [n], hkv, tdt, seed=0xC0FFEE + 1)
     q = torch.randn((layers, n, hq, D), device="cuda:0").to(tdt)
@@ -454,13 +452,6 @@ def main():
                                             "small launches use (the default picks the 16x16x32 kernel here)",
             "value": round(pre32["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre32["kernel_TFLOPs"], 2),
             "frac_of_mfma_peak": round(pre32["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre32["kernel_ms"] * 1e3, 2)}
-        pre1 = bench_prefill_c2(A, torch, max(20, args.steps // 4), max(5, args.warmup // 4), single_p=True)
-        log(f"[bench] prefill C2, bf16 with one operand per probability: {pre1['ms_per_step']:.3f} ms/step, "
-            f"{pre1['kernel_TFLOPs']:.1f} TFLOP/s kernel")
-        result["prefill_bf16_single_p"] = {
-            "workload": pre1["workload"] + ", option prefill_bf16_single_p=1 (adds ~1.5e-3 L2 error; not the default)",
-            "value": round(pre1["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre1["kernel_TFLOPs"], 2),
-            "frac_of_mfma_peak": round(pre1["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre1["kernel_ms"] * 1e3, 2)}
         probe = gemm_probe(torch)
         log(f"[bench] vendor bf16 GEMM 8192^3: {probe:.0f} TFLOP/s")
         result["mfma_peak_probe"] = {"what": "torch.matmul bf16 8192x8192x8192 (hipBLASLt)", "TFLOPs": round(probe, 1),

@@ -21,6 +21,11 @@
  *   k, v   : [n][num_kv_heads][head_dim]         kv_dtype
  *   scales : [num_kv_heads][head_dim]            float32 (int8 cache only)
  * Query head h reads KV head h / (num_q_heads / num_kv_heads).
+ * A bfloat16 cache keeps its K planes in bfloat16 and its V planes as IEEE half
+ * values, so that the probabilities multiply V with 11 significant bits on the
+ * fp16 matrix-core path: a bfloat16 value v is stored without loss for
+ * 2^-17 <= |v| <= 65504, larger magnitudes saturate at +-65504 and smaller ones
+ * round to the nearest multiple of 2^-24 (mi355_attn_kv_read returns what is stored).
  * Key j is visible to the query at absolute position p iff j <= p and, on a
  * layer with window W > 0, p - j < W.
  */
@@ -254,11 +259,6 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *                      workspace allocated on first use, [layers][rows][heads][parts]
  *                      x (head_dim + 2) floats, at most 258 MiB (else no split).
  *                      0: never; n > 0: n key blocks (of 32 keys) per work item
- *   "prefill_bf16_single_p" 0 (default): a bf16 prefill feeds each probability to
- *                      the P.V product as a high and a low bf16 part, which keeps the
- *                      result within the output format's own rounding; 1: one bf16
- *                      operand per probability (a third fewer MFMAs; adds ~1.5e-3
- *                      L2-relative error, the usual trade of bf16 attention kernels)
  */
 int mi355_attn_set_option(mi355_attn* handle, const char* name, int32_t value);
 

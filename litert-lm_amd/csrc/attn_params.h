@@ -21,6 +21,14 @@
 //   token-slice) of O^T = V^T . P^T, and their token order matches the
 //   accumulator layout in which S^T leaves the first MFMA, so P never moves
 //   between lanes.
+//
+//   V planes of a bfloat16 cache hold IEEE half (binary16) values: the
+//   probabilities that multiply V are numbers in [0, 1] that need mantissa, not
+//   range, and as half operands they enter O^T = V^T . P^T with 11 significant bits
+//   instead of 8 (one bfloat16 operand per probability costs ~1e-3 of relative
+//   error, two operands half the matrix-core rate). A bfloat16 value v converts
+//   without loss for 2^-17 <= |v| <= 65504; larger magnitudes saturate at +-65504
+//   and smaller ones round to the nearest multiple of 2^-24. K planes stay bfloat16.
 #ifndef LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_
 #define LITERT_LM_AMD_CSRC_ATTN_PARAMS_H_
 
@@ -139,7 +147,6 @@ struct PrefillArgs {
   // (global layers before windowed ones). use_order == 0: identity (more units than the table holds).
   const int32_t* host_window;  // host copy of layer_window (for the ordering), may be null
   int32_t use_order;
-  int32_t single_p;  // bf16: probabilities enter P.V as one bf16 operand (faster, ~1.5e-3 L2 error) instead of two
   // Key split (launches with fewer work items than compute units): a work item covers at most kchunk
   // key blocks of its tile, tiles with more blocks are cut into up to smax items whose unnormalised
   // fp32 accumulators and (max, sum) pairs go to ws_acc / ws_ml, [layer][row][head][smax] x head_dim
@@ -157,6 +164,7 @@ constexpr int kPrefillSchedInts = kPrefillQueues + 1;  // + count of workgroups 
 struct KvCopyArgs {
   uint8_t* cache;
   CacheGeom geom;
+  int32_t v_half;  // != 0: a bfloat16 cache, whose V planes hold IEEE half values (see the V plane note above)
   int32_t layer, seq, pos, n;
   void* k;  // [n][hkv][D] boundary layout (source for append, destination for read)
   void* v;

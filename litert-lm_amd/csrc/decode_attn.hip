@@ -148,29 +148,13 @@ __device__ __forceinline__ void qk_block(const u4 (&kreg)[D / 16], const u4* sm_
 // O^T += V^T . P^T for one block; p[T][i] pairs with token 16*T + 4*g + i.
 template <int KV, int D>
 __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)[KvT<KV>::VB / 16], f4 (&acc)[D / 16]) {
-  if constexpr (KV == kF16) {
+  if constexpr (KV == kF16 || KV == kBF16) {
+    // (the V planes of a bfloat16 cache hold IEEE half values, attn_params.h: both run on the fp16 MFMA)
     h8 pp;
 #pragma unroll
     for (int e = 0; e < 4; ++e) { pp[e] = (_Float16)p[0][e]; pp[4 + e] = (_Float16)p[1][e]; }
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) acc[db] = mfma16_f16(bit_cast<h8>(vreg[db]), pp, acc[db]);
-  } else if constexpr (KV == kBF16) {
-    // bf16 keeps 8 significant bits: P is fed as hi + lo parts (two MFMAs, the
-    // matrix cores are idle most of the time here) so that the probabilities
-    // enter P.V with ~16 bits instead of adding ~1e-3 of relative error.
-    b8 hi, lo;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      hi[e] = (__bf16)p[0][e];
-      hi[4 + e] = (__bf16)p[1][e];
-      lo[e] = (__bf16)(p[0][e] - (float)hi[e]);
-      lo[4 + e] = (__bf16)(p[1][e] - (float)hi[4 + e]);
-    }
-#pragma unroll
-    for (int db = 0; db < D / 16; ++db) {
-      acc[db] = mfma16_bf16(bit_cast<b8>(vreg[db]), hi, acc[db]);
-      acc[db] = mfma16_bf16(bit_cast<b8>(vreg[db]), lo, acc[db]);
-    }
   } else if constexpr (KV == kF32) {
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {

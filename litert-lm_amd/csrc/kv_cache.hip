@@ -13,8 +13,9 @@
 namespace mi355 {
 namespace {
 
-// One thread per 16-byte chunk of a source row. ESZ = element bytes.
-template <int ESZ, bool APPEND>
+// One thread per 16-byte chunk of a source row. ESZ = element bytes. VHALF: a bfloat16 cache,
+// whose V planes hold IEEE half values (attn_params.h): converted on the way in and out.
+template <int ESZ, bool APPEND, bool VHALF>
 __global__ void __launch_bounds__(256) kv_copy_kernel(const KvCopyArgs a) {
   constexpr int EPC = 16 / ESZ;
   const int D = a.geom.head_dim;
@@ -41,8 +42,10 @@ __global__ void __launch_bounds__(256) kv_copy_kernel(const KvCopyArgs a) {
     for (int e = 0; e < EPC; ++e) {
       uint8_t* dst = vplane + v_elem_offset(t, c * EPC + e, D, ESZ);
       if constexpr (ESZ == 4) *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src + 4 * e);
-      else if constexpr (ESZ == 2) *reinterpret_cast<uint16_t*>(dst) = *reinterpret_cast<const uint16_t*>(src + 2 * e);
-      else *dst = src[e];
+      else if constexpr (ESZ == 2) {
+        const uint16_t w = *reinterpret_cast<const uint16_t*>(src + 2 * e);
+        *reinterpret_cast<uint16_t*>(dst) = VHALF ? bf16_bits_to_half_bits(w) : w;
+      } else *dst = src[e];
     }
   } else {
     *reinterpret_cast<u4*>(kb) = *kc;
@@ -52,8 +55,10 @@ __global__ void __launch_bounds__(256) kv_copy_kernel(const KvCopyArgs a) {
     for (int e = 0; e < EPC; ++e) {
       const uint8_t* s = vplane + v_elem_offset(t, c * EPC + e, D, ESZ);
       if constexpr (ESZ == 4) *reinterpret_cast<uint32_t*>(dstb + 4 * e) = *reinterpret_cast<const uint32_t*>(s);
-      else if constexpr (ESZ == 2) *reinterpret_cast<uint16_t*>(dstb + 2 * e) = *reinterpret_cast<const uint16_t*>(s);
-      else dstb[e] = *s;
+      else if constexpr (ESZ == 2) {
+        const uint16_t w = *reinterpret_cast<const uint16_t*>(s);
+        *reinterpret_cast<uint16_t*>(dstb + 2 * e) = VHALF ? half_bits_to_bf16_bits(w) : w;
+      } else dstb[e] = *s;
     }
     *reinterpret_cast<u4*>(vb) = vw;
   }
@@ -65,9 +70,10 @@ hipError_t launch_copy(const KvCopyArgs& a, hipStream_t stream) {
   const int esz = a.geom.esize;
   const int64_t total = (int64_t)a.n * a.geom.hkv * (a.geom.head_dim / (16 / esz));
   const dim3 grid((unsigned)((total + 255) / 256));
-  if (esz == 4) hipLaunchKernelGGL((kv_copy_kernel<4, APPEND>), grid, dim3(256), 0, stream, a);
-  else if (esz == 2) hipLaunchKernelGGL((kv_copy_kernel<2, APPEND>), grid, dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((kv_copy_kernel<1, APPEND>), grid, dim3(256), 0, stream, a);
+  if (esz == 4) hipLaunchKernelGGL((kv_copy_kernel<4, APPEND, false>), grid, dim3(256), 0, stream, a);
+  else if (esz == 2 && a.v_half) hipLaunchKernelGGL((kv_copy_kernel<2, APPEND, true>), grid, dim3(256), 0, stream, a);
+  else if (esz == 2) hipLaunchKernelGGL((kv_copy_kernel<2, APPEND, false>), grid, dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((kv_copy_kernel<1, APPEND, false>), grid, dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -69,6 +69,18 @@ __device__ __forceinline__ void cvt_i8x16_to_h8x2(u4 w, h8& lo, h8& hi) {
   hi = bit_cast<h8>(b) - bias;
 }
 
+// bfloat16 bits -> the IEEE half that a V plane of a bfloat16 cache stores (exact for
+// 2^-17 <= |v| <= 65504, saturating above, nearest multiple of 2^-24 below), and back.
+__device__ __forceinline__ uint16_t bf16_bits_to_half_bits(uint16_t b) {
+  const float f = __uint_as_float((uint32_t)b << 16);
+  const _Float16 h = (_Float16)fminf(fmaxf(f, -65504.f), 65504.f);  // (NaN stays NaN)
+  return bit_cast<uint16_t>(h);
+}
+__device__ __forceinline__ uint16_t half_bits_to_bf16_bits(uint16_t hb) {
+  const float f = (float)bit_cast<_Float16>(hb);  // at most 11 significant bits; what came from a bfloat16 has 8
+  return bit_cast<uint16_t>((__bf16)f);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // tanh(y) = sign(y) * (1 - t) / (1 + t), t = exp(-2|y|): no overflow, no branch.

@@ -110,7 +110,6 @@ struct mi355_attn {
   DecodeTuning tuning;
   bool rowwise_prefill = false;  // force the row-wise prefill path (cross-checks)
   int prefill_workgroups = 0;    // 0 = one per CU
-  bool bf16_single_p = false;    // bf16 prefill: one MFMA operand per probability instead of a high and a low part
 };
 
 namespace {
@@ -353,7 +352,6 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.scale = h->cfg.scale;
     a.softcap = h->cfg.softcap;
     a.max_workgroups = h->prefill_workgroups;
-    a.single_p = h->bf16_single_p ? 1 : 0;
     a.rows16 = h->prefill_rows16;
     a.host_window = h->window.data();
     PrefillSplit split = plan_prefill_split(a, h->prefill_key_split);
@@ -594,6 +592,7 @@ int mi355_attn_kv_append(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos,
   KvCopyArgs a{};
   a.cache = h->cache;
   a.geom = h->geom;
+  a.v_half = h->cfg.kv_dtype == MI355_ATTN_BF16;
   a.layer = layer;
   a.seq = seq;
   a.pos = pos;
@@ -731,6 +730,7 @@ int mi355_attn_kv_read(mi355_attn* h, int32_t layer, int32_t seq, int32_t pos, i
   KvCopyArgs a{};
   a.cache = h->cache;
   a.geom = h->geom;
+  a.v_half = h->cfg.kv_dtype == MI355_ATTN_BF16;
   a.layer = layer;
   a.seq = seq;
   a.pos = pos;
@@ -813,8 +813,6 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   } else if (!strcmp(name, "prefill_key_split")) {
     if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_key_split = value;
-  } else if (!strcmp(name, "prefill_bf16_single_p")) {
-    h->bf16_single_p = value != 0;
   } else {
     return MI355_ATTN_INVALID_ARGUMENT;
   }

@@ -67,6 +67,15 @@ __device__ __forceinline__ void store_one(uint8_t* p, float a) {
   else *reinterpret_cast<__bf16*>(p) = (__bf16)a;
 }
 
+// A value-plane element: like store_one, except that a bfloat16 cache keeps its V planes as IEEE
+// half values (attn_params.h): the value is rounded to bfloat16 first, so that the cache holds
+// exactly what a bfloat16 row appended through the copy kernel would leave.
+template <int DT>
+__device__ __forceinline__ void store_value(uint8_t* p, float a) {
+  if constexpr (DT == kBF16) *reinterpret_cast<uint16_t*>(p) = bf16_bits_to_half_bits(bit_cast<uint16_t>((__bf16)a));
+  else store_one<DT>(p, a);
+}
+
 // round-half-away of x / scale, clamped to +-127; scale 0 stores 0
 __device__ __forceinline__ int quantise(float x, float scale) {
   const float inv = scale != 0.f ? 1.0f / scale : 0.f;
@@ -163,10 +172,10 @@ __global__ void __launch_bounds__(64 * kRowsPerWg) pre_attention_kernel(const Pr
       store_pair<KV>(plane + k_chunk_offset(t, d0 / EPC, kD, ESZ) + (d0 % EPC) * ESZ, x[0], x[1]);
       store_pair<KV>(plane + k_chunk_offset(t, d1 / EPC, kD, ESZ) + (d1 % EPC) * ESZ, x[2], x[3]);
     } else {
-      store_one<KV>(plane + v_elem_offset(t, d0, kD, ESZ), x[0]);
-      store_one<KV>(plane + v_elem_offset(t, d0 + 1, kD, ESZ), x[1]);
-      store_one<KV>(plane + v_elem_offset(t, d1, kD, ESZ), x[2]);
-      store_one<KV>(plane + v_elem_offset(t, d1 + 1, kD, ESZ), x[3]);
+      store_value<KV>(plane + v_elem_offset(t, d0, kD, ESZ), x[0]);
+      store_value<KV>(plane + v_elem_offset(t, d0 + 1, kD, ESZ), x[1]);
+      store_value<KV>(plane + v_elem_offset(t, d1, kD, ESZ), x[2]);
+      store_value<KV>(plane + v_elem_offset(t, d1 + 1, kD, ESZ), x[3]);
     }
   }
 }

@@ -386,33 +386,50 @@ def test_prefill_small_shapes(dt, hq, hkv, rows16):
 
 
 @ROWS16
-def test_prefill_bf16_one_operand_per_probability(rows16):
-    # option "prefill_bf16_single_p": P enters the P.V product as one bf16 value. Error beyond the output
-    # format's own rounding stays under 2e-3 (max-norm); with the output rounding the L2 figure is
-    # 2.0e-3 .. 2.5e-3 (the default, split, path stays under 2e-3, see err_of), bound here at 3e-3.
-    # A row that sees one key returns that key's V bit-exactly: the row sum is taken over the rounded values.
+def test_prefill_bf16_single_key_rows_are_exact(rows16):
+    # window 1: every row sees one key and must return that key's V row bit for bit (P = 1 exactly, the row
+    # sum is taken over the same rounded probabilities that multiply V)
     L, hq, hkv = 1024, 4, 1
-    windows = [0, 512, 1]
-    with make(len(windows), hq, hkv, L, 1, A.BF16, layer_window=windows) as at:
+    with make(1, hq, hkv, L, 1, A.BF16, layer_window=[1]) as at:
         at.set_option("prefill_rows16", rows16)
-        at.set_option("prefill_bf16_single_p", 1)
-        k, v = gen(161, L, hkv, D), gen(162, L, hkv, D)
-        for layer, w in enumerate(windows):
-            kr, vr = fill_seq(at, A.BF16, layer, 0, k, v)
-            for q_pos0, n in ((0, 1024), (129, 200), (1023, 1)):
-                qd, qr = dev(gen(2000 + n, n, hq, D), A.BF16)
-                out = torch.empty_like(qd)
-                at.prefill(layer, 0, q_pos0, n, qd, out)
-                torch.cuda.synchronize()
-                got = out.float().cpu().numpy()
-                ref = c_oracle.sdpa_f64(qr, kr, vr, D ** -0.5, q_pos0=q_pos0, window=w, kv_len=q_pos0 + n)
-                if w == 1:
-                    want = np.broadcast_to(vr[q_pos0:q_pos0 + n, 0][:, None, :], got.shape)
-                    assert np.array_equal(got, want)
-                    continue
-                beyond, l2 = orc.rel_err_beyond_bf16_rounding(got, ref), orc.l2_rel_err(got, ref)
-                say(f"single-P bf16 window={w} q_pos0={q_pos0} n={n}: beyond-rounding {beyond:.3e}, L2 {l2:.3e}")
-                assert beyond < TOL[A.BF16] and l2 < 3e-3
+        fill_seq(at, A.BF16, 0, 0, gen(161, L, hkv, D), gen(162, L, hkv, D))
+        ko = torch.empty((L, hkv, D), dtype=torch.bfloat16, device=DEV)
+        vo = torch.empty_like(ko)
+        at.kv_read(0, 0, 0, L, ko, vo)  # the values the planes hold (V magnitudes below 2^-17 are stored rounded)
+        vr = vo.float().cpu().numpy()
+        for q_pos0, n in ((0, 1024), (129, 200), (1023, 1)):
+            qd, _ = dev(gen(2000 + n, n, hq, D), A.BF16)
+            out = torch.empty_like(qd)
+            at.prefill(0, 0, q_pos0, n, qd, out)
+            torch.cuda.synchronize()
+            got = out.float().cpu().numpy()
+            want = np.broadcast_to(vr[q_pos0:q_pos0 + n, 0][:, None, :], got.shape)
+            assert np.array_equal(got, want)
+
+
+def test_bf16_value_planes_hold_half_precision_values():
+    """The V planes of a bfloat16 cache store IEEE half values: exact for 2^-17 <= |v| <= 65504, saturating
+    above, nearest multiple of 2^-24 below; K planes are bfloat16 as given."""
+    hkv, n = 1, 64
+    vals = np.zeros((n, hkv, D), np.float32)
+    rng = np.random.default_rng(5)
+    vals[:] = rng.standard_normal(vals.shape)
+    special = [2.0 ** -17, -(2.0 ** -17) * 1.9921875, 65280.0, -65280.0, 1.0e5, -3.0e38, 2.0 ** -20, -(2.0 ** -25) * 1.5,
+               2.0 ** -30, 0.0]
+    vals[0, 0, :len(special)] = special
+    with make(1, 4, hkv, n, 1, A.BF16) as at:
+        vd, vr = dev(vals, A.BF16)
+        at.kv_append(0, 0, 0, vd, vd)
+        ko, vo = torch.zeros_like(vd), torch.zeros_like(vd)
+        at.kv_read(0, 0, 0, n, ko, vo)
+        torch.cuda.synchronize()
+        assert torch.equal(ko, vd)  # keys: untouched
+        got = vo.float().cpu().numpy()
+        want = np.clip(vr, -65504.0, 65504.0).astype(np.float16).astype(np.float32)  # the half the plane holds ...
+        want = torch.from_numpy(want).bfloat16().float().numpy()                     # ... read back as bfloat16
+        assert np.array_equal(got, want)
+        exact = (np.abs(vr) >= 2.0 ** -17) & (np.abs(vr) <= 65504.0) | (vr == 0)
+        assert np.array_equal(got[exact], vr[exact]) and int((~exact).sum()) >= 5
 
 
 @ROWS16
