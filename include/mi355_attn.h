@@ -216,6 +216,23 @@ int mi355_attn_decode_layers(mi355_attn* handle, int32_t layer_begin, int32_t n_
                              void* out, int32_t num_splits, char** error_msg);
 
 /*
+ * mi355_attn_decode for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no
+ * counterpart in the reference. Same arguments, same kernels and bit-identical
+ * results, but the split-KV partials go to a fixed workspace that is part of the
+ * library image (8 MiB per GPU, held until the process ends) instead of the
+ * handle's growable one, and the call makes no hipMalloc / hipFree.
+ * Limits: the handle must use device pointers (host_io = 0, else
+ * kFailedPrecondition); batch x num_q_heads x num_splits <= 8192 partial results
+ * (an explicit num_splits beyond that is kResourceExhausted; with num_splits = 0
+ * the library chooses within the limit). All calls on one GPU share the
+ * workspace: calls that overlap in time on one GPU (two handles on two streams)
+ * race; calls queued on one stream do not.
+ */
+int mi355_attn_decode_noalloc(mi355_attn* handle, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,
+                              int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg);
+
+/*
  * Forgets the rows of sequence `seq` (seq < 0: all). Like
  * LlmLiteRtCompiledModelExecutor::Reset
  * (llm_litert_compiled_model_executor.cc:568-574) the cache memory itself is

@@ -90,6 +90,7 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_prefill.argtypes = [vp, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_prefill_layers.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_decode.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
+    L.mi355_attn_decode_noalloc.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
     L.mi355_attn_decode_layers.argtypes = [vp, i32, i32, i32p, i32p, i32, vp, vp, i32, errp]
     L.mi355_attn_reset.argtypes = [vp, i32, errp]
     L.mi355_attn_sync.argtypes = [vp, errp]
@@ -103,7 +104,7 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_cache_bytes.restype = ctypes.c_uint64
     L.mi355_attn_version.restype = ctypes.c_char_p
     for name in ("create", "kv_append", "kv_set_scales", "kv_read", "prefill", "prefill_layers", "decode",
-                 "decode_layers", "reset", "sync", "set_timing", "set_option"):
+                 "decode_layers", "decode_noalloc", "reset", "sync", "set_timing", "set_option"):
         getattr(L, "mi355_attn_" + name).restype = c
     _lib = L
     return L
@@ -243,6 +244,15 @@ class Attn:
             rc = lib().mi355_attn_decode_layers(self._h, layer, n_layers, sids, lens, batch, _ptr(q), _ptr(out),
                                                 num_splits, ctypes.byref(err))
         _check(rc, err)
+
+    def decode_noalloc(self, layer, kv_lens, q, out, seq_ids=None, num_splits=0, batch=None):
+        """mi355_attn_decode_noalloc: one layer, partials in the library's fixed workspace, no allocation."""
+        lens = kv_lens if isinstance(kv_lens, ctypes.Array) else _i32_array(kv_lens)
+        sids = seq_ids if isinstance(seq_ids, ctypes.Array) or seq_ids is None else _i32_array(seq_ids)
+        batch = len(lens) if batch is None else batch
+        err = ctypes.c_void_p()
+        _check(lib().mi355_attn_decode_noalloc(self._h, layer, sids, lens, batch, _ptr(q), _ptr(out), num_splits,
+                                               ctypes.byref(err)), err)
 
     # -- control
     def reset(self, seq=-1):

@@ -21,7 +21,19 @@
 
 using namespace mi355;
 
+// Workspace of mi355_attn_decode_noalloc: the split-KV partials of one call, (head_dim + 2) floats per
+// (layer, sequence, query head, partition), in device memory that exists from the moment the library
+// is loaded. Each GPU holds its own copy; host code reaches it only through the address that
+// hipGetSymbolAddress returns with that GPU current (resolved in mi355_attn_create), never through
+// the array's name.
+constexpr size_t kNoAllocSlots = 8192;  // partial slots: 8192 x 258 floats = 8.06 MiB per GPU
+constexpr int kNoAllocHeadDim = 256;
+static __device__ __align__(256) float scratch[kNoAllocSlots * (kNoAllocHeadDim + 2)];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {};  // [device]: address of `scratch` on that GPU, set once by create
 
 constexpr int kRingSlots = 64;
 constexpr int kMaxSplits = kMaxDecodeSplits;
@@ -231,9 +243,15 @@ void fill_inline_windows(const mi355_attn* h, DecodeArgs* a) {
   for (int i = 0; i < a->n_layers; ++i) a->inline_window[i] = h->window[a->layer_begin + i];
 }
 
+// no_alloc: the call may not allocate (mi355_attn_decode_noalloc): device pointers only, and the
+// partials go to this GPU's `scratch` instead of the handle's growable workspace.
 int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq_ids, const int32_t* kv_lens,
-                int batch, const void* q, void* out, int num_splits, char** error_msg) {
+                int batch, const void* q, void* out, int num_splits, char** error_msg, bool no_alloc = false) {
   if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (no_alloc && h->cfg.host_io)
+    return fail(error_msg, MI355_ATTN_FAILED_PRECONDITION,
+                "mi355_attn_decode_noalloc needs device pointers (the handle was created with host_io = 1, "
+                "whose staging buffers are allocated on demand)");
   if (int rc = check_layers(h, layer_begin, n_layers, error_msg)) return rc;
   if (!kv_lens || !q || !out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null kv_lens, q or out");
   if (batch < 1 || batch > h->cfg.max_seqs)
@@ -265,6 +283,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   }
   HIP_OR_RETURN(hipSetDevice(h->device));
   const int items = n_layers * batch;
+  const bool splits_chosen = num_splits == 0;
   if (num_splits == 0) {
     // About 1024 workgroups (four waves per CU saturate HBM; measured: 30 layers x 2 KV heads at 4096 tokens
     // run 8 % faster with 16-18 partitions than with 35, 16 layers x 64 sequences fastest without any split),
@@ -273,9 +292,29 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
     num_splits = std::max(1, std::min({want, (max_len + 63) / 64, 64}));
   }
   DecodeArgs a{};
-  if (num_splits > 1)
-    if (int rc = ensure_workspace(h, (size_t)items * h->cfg.num_q_heads * num_splits, error_msg)) return rc;
+  const size_t slots = (size_t)items * h->cfg.num_q_heads * num_splits;
+  if (no_alloc) {
+    // the library's own choice of partitions is trimmed to the workspace; an explicit count is an error
+    if (num_splits > 1 && slots > kNoAllocSlots) {
+      if (splits_chosen) {
+        num_splits = (int)(kNoAllocSlots / ((size_t)items * h->cfg.num_q_heads));
+      } else {
+        return fail(error_msg, MI355_ATTN_RESOURCE_EXHAUSTED,
+                    "mi355_attn_decode_noalloc: %d layers x %d sequences x %d query heads x %d partitions = %zu partial "
+                    "results, the fixed workspace holds %zu (pass fewer partitions, or 0 to let the library choose)",
+                    n_layers, batch, h->cfg.num_q_heads, num_splits, slots, kNoAllocSlots);
+      }
+      if (num_splits < 1) num_splits = 1;
+    }
+  } else if (num_splits > 1) {
+    if (int rc = ensure_workspace(h, slots, error_msg)) return rc;
+  }
   fill_decode_common(h, &a);
+  if (no_alloc) {
+    float* const base = g_scratch_ptr[h->device];  // this GPU's copy of `scratch`
+    a.ws_acc = base;
+    a.ws_ml = base + kNoAllocSlots * kNoAllocHeadDim;
+  }
   const size_t io_bytes = (size_t)items * h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
   const void* dq = nullptr;
   void* dout = nullptr;
@@ -497,6 +536,17 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
   };
   hipError_t e;
   if ((e = hipSetDevice(h->device)) != hipSuccess) return bail(MI355_ATTN_UNAVAILABLE, "hipSetDevice", e);
+  if (h->device >= kMaxDevices) {
+    int rc = fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "device %d: at most %d devices", h->device, kMaxDevices);
+    mi355_attn_destroy(h);
+    return rc;
+  }
+  if (!g_scratch_ptr[h->device]) {  // once per GPU, with that GPU current
+    float* p = nullptr;
+    if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch))) != hipSuccess || !p)
+      return bail(MI355_ATTN_INTERNAL, "hipGetSymbolAddress(scratch)", e);
+    g_scratch_ptr[h->device] = p;
+  }
   if (c->own_stream) {
     if ((e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking)) != hipSuccess)
       return bail(MI355_ATTN_INTERNAL, "hipStreamCreate", e);
@@ -761,6 +811,12 @@ int mi355_attn_decode_layers(mi355_attn* h, int32_t layer_begin, int32_t n_layer
                              const int32_t* kv_lens, int32_t batch, const void* q, void* out, int32_t num_splits,
                              char** error_msg) {
   return decode_impl(h, layer_begin, n_layers, seq_ids, kv_lens, batch, q, out, num_splits, error_msg);
+}
+
+int mi355_attn_decode_noalloc(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,
+                              int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg) {
+  static_assert(kNoAllocHeadDim == 256, "the workspace is laid out for the one head_dim the library builds");
+  return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg, /*no_alloc=*/true);
 }
 
 int mi355_attn_reset(mi355_attn* h, int32_t seq, char** error_msg) {
