@@ -48,7 +48,6 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKeysPerBlock = 32;  // one V block of a 16-bit cache = two K tiles
-constexpr float kNoKey = -1.0e30f;  // reference maximum of a row before its first visible key (16x16x32 kernel)
 constexpr float kRescaleSlack = 8.f;  // log2 units a score may exceed the reference max before it is moved
 
 template <int T>
@@ -98,25 +97,6 @@ constexpr int kWaitVm8 = 0x0F78;  // all but the 8 most recent ones
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
-// LDS operand reads whose waits the code places itself. The compiler waits for every outstanding LDS
-// operation (lgkmcnt(0)) in front of the first use of any one of them while a transfer into LDS is
-// under way, i.e. also for the read issued a moment ago; with the reads in inline assembly it does not
-// know of them, and lds_wait<N>(x) in front of the use of x says "all but the N most recent LDS
-// operations of this wave have returned" (they return in order). The "+v" operand ties the wait to the
-// register it guards, so nothing that uses x can be scheduled above it.
-template <class V>
-__device__ __forceinline__ void lds_read16(V& dst, unsigned lds_addr, int offset) {
-  static_assert(sizeof(V) == 16, "one 16-byte operand per lane");
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(lds_addr), "n"(offset));
-}
-template <int N, class V>
-__device__ __forceinline__ void lds_wait(V& x) {
-  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
-}
-__device__ __forceinline__ unsigned lds_address(const void* p) {
-  return (unsigned)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void*)p);
-}
-
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.
 template <int... Is, class F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
@@ -630,25 +610,16 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
 // straight in the cache planes' order (the layout the decode kernel uses), every
 // operand read from LDS feeding two MFMAs (one per sub-tile). A workgroup needs
 // 80 KiB of LDS (K ring of three blocks, V ring of two) and 256 registers per
-// wave, so two workgroups share a CU, two waves a SIMD.
-//
-// The key loop is software-pipelined inside the wave, half a block (16 keys) deep. Iteration i:
-//   first half-step:  S^T of the keys 16 .. 31 of block i on the matrix cores, and under those 16
-//                     MFMAs the exponentials of its keys 0 .. 15 (8 per lane: one multiply-add, one
-//                     exp2, half a packed conversion each) on the vector ALU;
-//   second half-step: S^T of the keys 0 .. 15 of block i+1 beside the exponentials of the keys
-//                     16 .. 31 of block i;
-//   barrier (K(i+2) and V(i) have landed for everybody), K(i+3) and V(i+1) requested;
-//   O^T += V(i)^T . P(i)^T (32 MFMAs), the row sums (two rounded probabilities per instruction)
-//   beside it.
-// So only two half-blocks of scores are ever in registers (16 per lane, what the unpipelined loop
-// needs for one block), which leaves room for four operand reads in flight.
-// The exponentials take the running reference maximum as it stands: it only moves when a score
-// exceeds it by kRescaleSlack (2^8 as a probability, harmless in half precision), which the wave
-// learns by a vote right after a half-block's scores are complete, before their exponentials start;
-// the accumulators are rescaled there, and with them the probabilities of the block's first half
-// when they are still waiting for their product with V. The two instruction streams are dealt out
-// in program order, one scheduling region per MFMA.
+// wave, so two workgroups share a CU, two waves a SIMD: they work on different
+// items and fill each other's stalls. The probabilities enter P.V as IEEE half
+// operands for both cache types (the V planes of a bfloat16 cache hold half values,
+// attn_params.h), so P.V always runs on the fp16 MFMA.
+// (Measured and not kept: the same loop software-pipelined inside the wave - scores of
+// the next half-block and the exponentials of the current one dealt out in one
+// instruction stream, operand reads with counted waits, one continuous read stream
+// across the phases - is 3 to 10 % slower on the 26-layer launch: the exponentials
+// were already hidden by the other wave of the SIMD, and what the hand-placed order
+// adds in scheduling regions and waits costs more than the phases' ramps it removes.)
 constexpr int kWaves16 = 4;
 constexpr int kRows16 = 16;
 constexpr int kSub16 = 2;       // sub-tiles of 16 query positions per wave
@@ -659,6 +630,7 @@ template <int D>
 constexpr int prefill16_lds_bytes() { return (kKStages16 + kVStages16) * 64 * D; }  // 80 KiB: two workgroups fill a CU's LDS
 
 template <int DT, int D, int HPB, bool CAP>
+
 __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
@@ -668,7 +640,7 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
   constexpr int NL = D / 16;  // 16-channel tiles of O^T
   constexpr int kBlockBytes = 64 * D;
   constexpr int kXfers = 16 / kWaves16;
-  auto mfma_qk = [](vec8 x, vec8 y, f4 z) {
+  auto mfma = [](vec8 x, vec8 y, f4 z) {
     if constexpr (DT == kF16) return mfma16_f16(x, y, z);
     else return mfma16_bf16(x, y, z);
   };
@@ -684,7 +656,6 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
-  const unsigned lane16 = (unsigned)lane * 16u;
   const int hblocks = a.group / HPB;
   const int per_layer = a.geom.hkv * hblocks;
   const int units = a.n_layers * per_layer;
@@ -694,8 +665,7 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
   bool first_draw = true;
   const int smax = a.kchunk > 0 ? a.smax : 1;
   const float softcap = a.softcap;
-  // (wave-uniform: kept in a scalar register)
-  const float c = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(CAP ? 1.f : a.scale * kLog2e)));
+  const float c = CAP ? 1.f : a.scale * kLog2e;
   const int pos_end = a.q_pos0 + a.n;
 
   struct Item { int li, kvh, hb, tile, part, layer, window, wg_pos0, kb_lo, nblk_tile; };
@@ -764,25 +734,21 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
     auto fetch = [&](const uint8_t* plane, uint8_t* ring, int stages, int i) {
 #pragma unroll
       for (int t = 0; t < kXfers; ++t) {
-        // (scalar base + one 32-bit lane offset: no 64-bit address per lane to keep in registers)
         const int off = (wave + kWaves16 * t) * 1024;
-        const uint8_t* src = plane + (int64_t)(kb_lo + i) * kBlockBytes + off;
+        const uint8_t* src = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16 + off;
         uint8_t* dst = ring + (i % stages) * kBlockBytes + off;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (size_t)lane16),
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
       }
     };
-    // Ring protocol, one barrier per block, all requests behind it. After the barrier of iteration i
-    // every wave has finished phase A of i (the last reader of K(i+1)... of K(i) was phase A of i-1)
-    // and phase B of i-1 (the last reader of V(i-1)): K(i+3) goes into the stage of K(i), V(i+1)
-    // into the stage of V(i-1). Both are first read behind the barrier of iteration i+1 (K(i+3) in
-    // phase A of i+2), in front of which every wave waits for all of its own transfers: each one has
-    // a whole iteration to land.
-    // (K(2) waits for the first barrier: its stage ends in the ticket words, which every wave must have read)
+    // Ring protocol, one barrier per block. Iteration i: K(i + 2) is asked for at
+    // the top (its stage held K(i - 1), read before the middle barrier of i - 1);
+    // scores and softmax of block i; every wave waits for its share of V(i) (asked
+    // for in the middle of i - 1; K(i + 1), older still, has then landed too);
+    // barrier; V(i + 1) is asked for (its stage held V(i - 1)); P.V of block i.
     fetch(kplane, sm_k, kKStages16, 0);
     fetch(vplane, sm_v, kVStages16, 0);
     if (nblk > 1) fetch(kplane, sm_k, kKStages16, 1);
-    asm volatile("" ::: "memory");  // the query loads are issued behind the transfers: the counted wait below relies on it
 
     // Q^T operands: lane (n, g) holds, for sub-tile u and step j, channels 32 j + 8 g .. + 7 of query my_pos0 + 16 u + n
     vec8 q[kSub16][NJ];
@@ -794,202 +760,112 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       for (int j = 0; j < NJ; ++j) q[u][j] = *reinterpret_cast<const vec8*>(qrow + 32 * j + 8 * g);
     }
     f4 acc[kSub16][NL];
-    float l_run[kSub16];  // row sums, this lane's share (keys 4 g .. 4 g + 3 of every 16)
 #pragma unroll
-    for (int u = 0; u < kSub16; ++u) {
+    for (int u = 0; u < kSub16; ++u)
 #pragma unroll
       for (int i = 0; i < NL; ++i) acc[u][i] = f4{0.f, 0.f, 0.f, 0.f};
-      l_run[u] = 0.f;
-    }
-    // Reference maximum per query (exp2 domain). A row that has not met a visible key yet holds kNoKey
-    // (finite, so that -inf scores minus the reference stay -inf and exp2 gives 0 without a special case).
-    float m_run[kSub16];
+    float m_run[kSub16], l_run[kSub16];
 #pragma unroll
-    for (int u = 0; u < kSub16; ++u) m_run[u] = kNoKey;
+    for (int u = 0; u < kSub16; ++u) { m_run[u] = -INFINITY; l_run[u] = 0.f; }
     const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
     const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
+    // K(0) has to be there for everybody (the query loads, issued last, may still be under way;
+    // the compiler waits for those where it needs them)
+    __builtin_amdgcn_s_waitcnt(wait_vm(kSub16 * NJ));
+    lds_barrier();
 
-    u4 pw[kSub16];  // the probabilities of a block as half-precision MFMA operands: word 2 T + e / 2 of sub-tile u
-    // Soft cap and visibility of the raw scores of half-block (b, T), keys key0 .. key0 + 15 (wave-uniform
-    // branches: only the half-blocks on the diagonal and at the window's edge hold keys that some row does not see).
-    // score sc[u][e]: key key0 + 4 g + e against query my_pos0 + 16 u + n
-    auto prepare = [&](f4 (&sc)[kSub16], int b, int T) {
-      const int key0 = (kb_lo + b) * kKeysPerBlock + 16 * T;
-      if constexpr (CAP) {
+    for (int i = 0; i < nblk; ++i) {
+      const bool more_k = i + 2 < nblk, more_v = i + 1 < nblk;
+      if (more_k) fetch(kplane, sm_k, kKStages16, i + 2);
+      const uint8_t* kb = sm_k + (i % kKStages16) * kBlockBytes + lane * 16;
+      const uint8_t* vb = sm_v + (i % kVStages16) * kBlockBytes + lane * 16;
+      f4 sc[kSub16][2];
 #pragma unroll
-        for (int u = 0; u < kSub16; ++u)
+      for (int u = 0; u < kSub16; ++u)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) sc[u][e] = (softcap * kLog2e) * fast_tanh(sc[u][e] * (a.scale / softcap));
-      }
-      const bool all_vis = key0 + 15 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim;
-      if (!all_vis) {
+        for (int T = 0; T < 2; ++T) sc[u][T] = f4{0.f, 0.f, 0.f, 0.f};
+      {
+        // operand reads run kOpAhead steps ahead of the MFMAs that use them (an LDS read takes longer
+        // than the two MFMAs of a step)
+        auto k_at = [&](int step) { return *reinterpret_cast<const vec8*>(kb + (step & 1) * (16 * D * 2) + (step >> 1) * 1024); };
+        vec8 kop[kOpAhead];
 #pragma unroll
-        for (int u = 0; u < kSub16; ++u) {
-          const int my_pos = my_pos0 + kRows16 * u + n;
+        for (int st = 0; st < kOpAhead; ++st) kop[st] = k_at(st);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) sc[u][e] = (unsigned)(my_pos - (key0 + 4 * g + e)) < wlim ? sc[u][e] : -INFINITY;
+        for (int st = 0; st < 2 * NJ; ++st) {
+          const int j = st >> 1, T = st & 1;
+#pragma unroll
+          for (int u = 0; u < kSub16; ++u) sc[u][T] = mfma(kop[st % kOpAhead], q[u][j], sc[u][T]);
+          if (st + kOpAhead < 2 * NJ) kop[st % kOpAhead] = k_at(st + kOpAhead);
         }
       }
-    };
-    // The maxima of a half-block (exp2 domain) against the running references: only when some lane has seen
-    // a score above its reference by more than the slack do the four lanes of a query compare notes and
-    // the references (and with them the accumulators) move. Rare after the first blocks.
-    // PENDING: the probabilities of the block's first half-block are in pw (words 0 and 1), computed under
-    // the old references and not added yet: they are rescaled with the accumulators.
-    auto move_reference = [&](const f4 (&sc)[kSub16], auto pending_tag) {
-      constexpr bool PENDING = decltype(pending_tag)::value;
-      float bm[kSub16];
-      bool over = false;
+      // score sc[u][T][e]: key key0 + 16 T + 4 g + e against query my_pos0 + 16 u + n
+      const int key0 = (kb_lo + i) * kKeysPerBlock;
+      const bool all_vis = key0 + kKeysPerBlock - 1 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim;
+      h8 p_hi[kSub16];
 #pragma unroll
       for (int u = 0; u < kSub16; ++u) {
-        bm[u] = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(sc[u][0], sc[u][1]), sc[u][2]), sc[u][3]) * c;
-        over = over || bm[u] > m_run[u] + kRescaleSlack;
-      }
-      if (!__any(over)) return;
+        const int my_pos = my_pos0 + kRows16 * u + n;
+        float bm = -INFINITY;
 #pragma unroll
-      for (int u = 0; u < kSub16; ++u) {
-        float bx = wave_xor_max(bm[u], 16);
-        bx = wave_xor_max(bx, 32);
-        const float m_new = bx > m_run[u] + kRescaleSlack ? bx : m_run[u];
-        const float alpha = fast_exp2(m_run[u] - m_new);  // (from kNoKey: 0, and the accumulators are still 0)
+        for (int T = 0; T < 2; ++T)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = sc[u][T][e];
+            if constexpr (CAP) x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
+            if (!all_vis) x = (unsigned)(my_pos - (key0 + 16 * T + 4 * g + e)) < wlim ? x : -INFINITY;
+            sc[u][T][e] = x;
+            bm = fmaxf(bm, x);
+          }
+        bm *= c;
+        // The four lanes of a query compare notes only when one of them has seen a score that
+        // exceeds the reference by more than the slack: rare after the first blocks.
+        if (__any(bm > m_run[u] + kRescaleSlack)) {
+          bm = wave_xor_max(bm, 16);
+          bm = wave_xor_max(bm, 32);
+        }
+        const float m_new = bm > m_run[u] + kRescaleSlack ? bm : m_run[u];
+        const float alpha = (m_run[u] == -INFINITY) ? 1.f : fast_exp2(m_run[u] - m_new);
+        const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
         m_run[u] = m_new;
+        float lsum = 0.f;
+        {
+#pragma unroll
+          for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float pv = fast_exp2(fmaf(sc[u][T][e], c, neg_m));
+              p_hi[u][4 * T + e] = (_Float16)pv;
+              lsum += pv;
+            }
+        }
+        l_run[u] = l_run[u] * alpha + lsum;
         if (__any(alpha != 1.f)) {
 #pragma unroll
           for (int db = 0; db < NL; ++db) acc[u][db] *= alpha;
-          l_run[u] *= alpha;
-          if constexpr (PENDING) {
-            const h2 a2 = {(_Float16)alpha, (_Float16)alpha};
-#pragma unroll
-            for (int w = 0; w < 2; ++w) pw[u][w] = bit_cast<unsigned>(bit_cast<h2>(pw[u][w]) * a2);
-          }
         }
       }
-    };
-
-    // K(0), V(0), K(1) are there for everybody; the kSub16 * NJ query loads, issued behind them, may
-    // still be under way (the compiler waits for those where it needs them). The memory clobbers keep
-    // the loads between the two statements, so the count is exact.
-    static_assert(kSub16 * NJ == 16, "the counted wait below");
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    lds_barrier();
-    if (nblk > 2) fetch(kplane, sm_k, kKStages16, 2);
-
-    f4 sc_a[kSub16], sc_b[kSub16];  // scores of two consecutive half-blocks: one in the softmax, one being summed
-
-    // S^T of half-block (b, T) into sc: 16 MFMAs (8 channel steps x 2 sub-tiles), K operands kOpAhead
-    // reads ahead; piece(k) is called once per MFMA, k = 0 .. 15, for what runs on the vector ALU beside it.
-    auto scores = [&](f4 (&sc)[kSub16], int b, int T, auto&& piece) {
-      const unsigned kb = lds_address(sm_k + (b % kKStages16) * kBlockBytes) + T * (16 * D * 2) + lane16;
-      vec8 kop[kOpAhead];
-      static_for<kOpAhead>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
-        lds_read16(kop[j], kb, j * 1024);
-      });
-      static_for<NJ>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
-        constexpr int younger = NJ - 1 - j < kOpAhead - 1 ? NJ - 1 - j : kOpAhead - 1;  // reads issued behind this one
-        static_for<kSub16>([&](auto uc) {
-          constexpr int u = decltype(uc)::value;
-          __builtin_amdgcn_sched_barrier(0);
-          if constexpr (u == 0) lds_wait<younger>(kop[j % kOpAhead]);
-          if constexpr (j == 0) sc[u] = mfma_qk(kop[j % kOpAhead], q[u][j], f4{0.f, 0.f, 0.f, 0.f});
-          else sc[u] = mfma_qk(kop[j % kOpAhead], q[u][j], sc[u]);
-          piece(std::integral_constant<int, kSub16 * j + u>{});
-        });
-        if constexpr (j + kOpAhead < NJ) lds_read16(kop[j % kOpAhead], kb, (j + kOpAhead) * 1024);
-      });
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    // The 8 exponentials of a half-block T (prepared scores in sc) as 16 slots, one per MFMA of the scores
-    // computed beside them, so that no vector-ALU instruction waits for the one right in front of it:
-    // slot 2 k holds the multiply-add of score k = (u, e) = (k / 4, k % 4) and the packed conversion of the
-    // pair finished before, slot 2 k + 1 the exp2 of score k; exponential_drain packs the last pair.
-    float ex_x = 0.f, ex_y[2] = {0.f, 0.f};
-    auto pack_pair = [&](auto Tc, auto kc) {  // scores k - 1, k (k odd) -> word 2 T + e / 2 of sub-tile u
-      constexpr int T = decltype(Tc)::value, k = decltype(kc)::value;
-      constexpr int u = k / 4, e = k % 4;
-      const h2 pair = {(_Float16)ex_y[0], (_Float16)ex_y[1]};
-      pw[u][2 * T + e / 2] = bit_cast<unsigned>(pair);
-      asm volatile("" : "+v"(pw[u][2 * T + e / 2]));
-    };
-    auto exponential_slot = [&](const f4 (&sc)[kSub16], auto Tc, auto sc_) {
-      constexpr int slot = decltype(sc_)::value;
-      constexpr int k = slot / 2;
-      constexpr int u = k / 4, e = k % 4;
-      if constexpr (slot % 2 == 0) {
-        if constexpr (k >= 2 && k % 2 == 0) pack_pair(Tc, std::integral_constant<int, k - 1>{});
-        ex_x = fmaf(sc[u][e], c, -m_run[u]);
-        asm volatile("" : "+v"(ex_x));
-      } else {
-        ex_y[k & 1] = fast_exp2(ex_x);
-        asm volatile("" : "+v"(ex_y[k & 1]));
-      }
-    };
-    auto exponential_drain = [&](auto Tc) { pack_pair(Tc, std::integral_constant<int, 7>{}); };
-    // Row sums over the rounded probabilities (the values that multiply V): two per instruction, half
-    // precision in, single precision out. Word w (0 .. 3) of sub-tile u.
-    typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));
-    const fp16x2 one2 = {(__fp16)1.f, (__fp16)1.f};
-    auto row_sum = [&](int u, int w) {
-      l_run[u] = __builtin_amdgcn_fdot2(bit_cast<fp16x2>(pw[u][w]), one2, l_run[u], false);
-      asm volatile("" : "+v"(l_run[u]));
-    };
-    constexpr std::integral_constant<int, 0> half0{};
-    constexpr std::integral_constant<int, 1> half1{};
-
-    // ---- half-block (0, 0): scores, preparation, first reference
-    scores(sc_a, 0, 0, [](auto) {});
-    prepare(sc_a, 0, 0);
-    move_reference(sc_a, std::false_type{});
-
-    // One iteration: the prepared scores of half-block (i, 0) are in sc_a and the references cover them.
-    // NEXT: block i + 1 exists.
-    auto iteration = [&](int i, auto next_tag) {
-      constexpr bool NEXT = decltype(next_tag)::value;
-      // ---- first half-step: scores of (i, 1) beside the exponentials of (i, 0)
-      scores(sc_b, i, 1, [&](auto kc) { exponential_slot(sc_a, half0, kc); });
-      exponential_drain(half0);
-      prepare(sc_b, i, 1);
-      move_reference(sc_b, std::true_type{});
-      // ---- second half-step: scores of (i + 1, 0) beside the exponentials of (i, 1)
-      if constexpr (NEXT) {
-        scores(sc_a, i + 1, 0, [&](auto kc) { exponential_slot(sc_b, half1, kc); });
-      } else {
-        static_for<16>([&](auto kc) { exponential_slot(sc_b, half1, kc); });
-      }
-      exponential_drain(half1);
-      // every transfer this wave has asked for has landed: V(i) and K(i + 2) among them
-      __builtin_amdgcn_s_waitcnt(kWaitVm0);
+      // this wave's share of V(i) (and of K(i + 1)) has landed; K(i + 2) may be under way
+      if (more_k) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
       lds_barrier();
-      if (i + 3 < nblk) fetch(kplane, sm_k, kKStages16, i + 3);
-      if (i + 1 < nblk) fetch(vplane, sm_v, kVStages16, i + 1);
-      if constexpr (NEXT) prepare(sc_a, i + 1, 0);
-      // ---- O^T += V(i)^T . P(i)^T, the row sums beside it
-      const unsigned vb = lds_address(sm_v + (i % kVStages16) * kBlockBytes) + lane16;
-      h8 vop[kOpAhead];
-      static_for<kOpAhead>([&](auto sc_) {
-        constexpr int st = decltype(sc_)::value;
-        lds_read16(vop[st], vb, st * 1024);
-      });
-      static_for<NL>([&](auto dbc) {
-        constexpr int db = decltype(dbc)::value;
-        constexpr int younger = NL - 1 - db < kOpAhead - 1 ? NL - 1 - db : kOpAhead - 1;
-        static_for<kSub16>([&](auto uc) {
-          constexpr int u = decltype(uc)::value;
-          __builtin_amdgcn_sched_barrier(0);
-          if constexpr (u == 0) lds_wait<younger>(vop[db % kOpAhead]);
-          acc[u][db] = mfma16_f16(vop[db % kOpAhead], bit_cast<h8>(pw[u]), acc[u][db]);
-          if constexpr (db < 4) row_sum(u, db);
-        });
-        if constexpr (db + kOpAhead < NL) lds_read16(vop[db % kOpAhead], vb, (db + kOpAhead) * 1024);
-      });
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (NEXT) move_reference(sc_a, std::false_type{});
-    };
-    constexpr std::true_type yes{};
-    constexpr std::false_type no{};
-    for (int i = 0; i + 1 < nblk; ++i) iteration(i, yes);
-    iteration(nblk - 1, no);
+      if (more_v) fetch(vplane, sm_v, kVStages16, i + 1);
+      {
+        h8 vop[kOpAhead];
+#pragma unroll
+        for (int st = 0; st < kOpAhead; ++st) vop[st] = *reinterpret_cast<const h8*>(vb + st * 1024);
+#pragma unroll
+        for (int db = 0; db < NL; ++db) {
+#pragma unroll
+          for (int u = 0; u < kSub16; ++u) {
+            acc[u][db] = mfma16_f16(vop[db % kOpAhead], p_hi[u], acc[u][db]);
+          }
+          if (db + kOpAhead < NL) vop[db % kOpAhead] = *reinterpret_cast<const h8*>(vb + (db + kOpAhead) * 1024);
+        }
+      }
+      // (no barrier here: the next one, in the middle of iteration i + 1, is passed only when every
+      // wave is done with this P.V, and V(i)'s stage is written no earlier than that)
+    }
 
     // ---- store: lane (n, g) holds channels 16 db + 4 g .. + 3 of query my_pos0 + 16 u + n
 #pragma unroll
@@ -1008,8 +884,8 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       }
       if (!split_tile) {
         // Whole rows through LDS (the K ring is idle: every wave has passed the last barrier of the
-        // loop, behind which nobody reads K; each wave has a patch of its own, 16 rows padded to 528
-        // bytes, below the ticket), then two 512-byte rows per store instruction.
+        // loop; each wave has a patch of its own, 16 rows padded to 528 bytes, below the ticket), then
+        // two 512-byte rows per store instruction.
         constexpr int kRowStride = 2 * D + 16;
         static_assert(kWaves16 * kRows16 * kRowStride <= kKStages16 * kBlockBytes - 16, "patches below the ticket");
         uint8_t* const patch = sm_k + wave * (kRows16 * kRowStride);
