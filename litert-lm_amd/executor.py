@@ -57,6 +57,7 @@ def lib():
         for n in ("hle_current_step", "hle_vocab_size", "hle_max_num_tokens", "hle_num_runs"):
             getattr(L, n).argtypes = [vp]
         L.hle_reset.argtypes = [vp, errp]
+        L.hle_fill_vision_embeddings.argtypes = [vp, i32, errp]
         L.hle_backend_name.argtypes = [vp]
         L.hle_backend_name.restype = ctypes.c_char_p
         L.hle_get_run.argtypes = [vp, i32, i32p, i32p, i32p, i32]
@@ -167,6 +168,11 @@ class HipLlmExecutor:
     def reset(self):
         err = ctypes.c_void_p()
         _check(lib().hle_reset(self._h, ctypes.byref(err)), err)
+
+    def fill_vision_embeddings(self, image_index: int = 0):
+        """LlmExecutorBase::FillVisionEmbeddings with empty vision data (not implemented by this executor)."""
+        err = ctypes.c_void_p()
+        _check(lib().hle_fill_vision_embeddings(self._h, image_index, ctypes.byref(err)), err)
 
     def runs(self):
         """[(kind, tokens, positions)] of every forward pass since the last reset."""

@@ -103,9 +103,13 @@ int hle_current_step(void* h) { return *static_cast<HipLlmExecutor*>(h)->GetCurr
 int hle_vocab_size(void* h) { return *static_cast<HipLlmExecutor*>(h)->GetVocabSize(); }
 int hle_max_num_tokens(void* h) { return static_cast<HipLlmExecutor*>(h)->GetExecutorSettings()->GetMaxNumTokens(); }
 int hle_reset(void* h, char** err) { return Finish(static_cast<HipLlmExecutor*>(h)->Reset(), err); }
+// The base class's default: no vision input in this executor.
+int hle_fill_vision_embeddings(void* h, int32_t image_index, char** err) {
+  return Finish(static_cast<HipLlmExecutor*>(h)->FillVisionEmbeddings(ExecutorVisionData(), image_index), err);
+}
 const char* hle_backend_name(void* h) {
   static thread_local std::string name;
-  name = static_cast<HipLlmExecutor*>(h)->ExecutorBackendName();
+  name = std::string(static_cast<HipLlmExecutor*>(h)->ExecutorBackendName());
   return name.c_str();
 }
 

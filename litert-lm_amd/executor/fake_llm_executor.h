@@ -70,7 +70,7 @@ class FakeLlmExecutor : public LlmExecutorBase {
     return logits;
   }
 
-  std::string ExecutorBackendName() const override { return "FakeLlmExecutorBackend"; }
+  string_view ExecutorBackendName() const override { return "FakeLlmExecutorBackend"; }
   StatusOr<int> GetVocabSize() override { return vocab_size_; }
   StatusOr<int> GetCurrentStep() const override { return current_step_; }
   StatusOr<LlmExecutorSettings> GetExecutorSettings() const override { return settings_; }

@@ -55,7 +55,7 @@ class HipLlmExecutor : public LlmExecutorBase {
   Status Decode(TensorBuffer& output_tokens) override;
   Status Decode(const ExecutorInputs& inputs, TensorBuffer& output_logits) override;
   StatusOr<TensorBuffer> DecodeLogits(const ExecutorInputs& inputs) override;
-  std::string ExecutorBackendName() const override { return "MI355X HIP attention"; }
+  string_view ExecutorBackendName() const override { return "MI355X HIP attention"; }
   StatusOr<int> GetVocabSize() override { return layers_->VocabSize(); }
   // What the caller expects: tokens handed in so far, the deferred one included
   // (llm_litert_compiled_model_executor.h:95-97).

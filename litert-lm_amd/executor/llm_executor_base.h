@@ -1,7 +1,9 @@
 // The executor interface this build plugs into: same methods, argument meaning
 // and default behaviour (UnimplementedError naming the backend) as
-// LlmExecutorBase in runtime/executor/llm_executor_base.h:33-121. The vision
-// entry point is omitted with the vision types.
+// LlmExecutorBase in runtime/executor/llm_executor_base.h:33-121, so that a
+// class derived from this one compiles against the reference's header once the
+// stand-in types (Status, string_view, TensorBuffer) are swapped for absl's and
+// LiteRT's.
 #ifndef LITERT_LM_AMD_EXECUTOR_LLM_EXECUTOR_BASE_H_
 #define LITERT_LM_AMD_EXECUTOR_LLM_EXECUTOR_BASE_H_
 
@@ -37,15 +39,21 @@ class LlmExecutorBase {
     (void)inputs;
     return Unimplemented("Decode for logits output");
   }
-  virtual std::string ExecutorBackendName() const = 0;
+  virtual string_view ExecutorBackendName() const = 0;
   virtual StatusOr<int> GetVocabSize() { return Unimplemented("GetVocabSize"); }
   virtual StatusOr<int> GetCurrentStep() const { return Unimplemented("GetCurrentStep"); }
   virtual StatusOr<LlmExecutorSettings> GetExecutorSettings() const { return Unimplemented("GetExecutorSettings"); }
+  // Vision embeddings of image `image_index` for the prefill that follows (llm_executor_base.h:108).
+  virtual Status FillVisionEmbeddings(const ExecutorVisionData& vision_input, int image_index) {
+    (void)vision_input;
+    (void)image_index;
+    return Unimplemented("FillVisionEmbeddings");
+  }
   virtual Status Reset() { return Unimplemented("Reset"); }
 
  private:
   Status Unimplemented(const char* what) const {
-    return UnimplementedError(std::string(what) + " not implemented for backend: " + ExecutorBackendName());
+    return UnimplementedError(std::string(what) + " not implemented for backend: " + std::string(ExecutorBackendName()));
   }
 };
 

@@ -1,7 +1,8 @@
 // Argument types of the executor interface, text path only. Mirrors the parts
 // of runtime/executor/llm_executor_io_types.h that the hot path reads:
 // ExecutorInputs::GetTextTokenIdsPtr (:172-213) and ExecutorPrefillParams
-// (:217-250). Vision and audio inputs are outside this build.
+// (:217-250). Vision data is carried as a type only (the executor interface names
+// it); audio inputs are outside this build.
 #ifndef LITERT_LM_AMD_EXECUTOR_LLM_EXECUTOR_IO_TYPES_H_
 #define LITERT_LM_AMD_EXECUTOR_LLM_EXECUTOR_IO_TYPES_H_
 
@@ -27,13 +28,37 @@ class ExecutorTextData {
   TensorBuffer token_ids_;
 };
 
+// Vision embeddings `[vision_tokens, model_dim]` and per-layer embeddings `[layers, vision_tokens, dim]`
+// (llm_executor_io_types.h:81-116). No executor of this build consumes them: the type exists so that
+// LlmExecutorBase::FillVisionEmbeddings has the reference's signature.
+class ExecutorVisionData {
+ public:
+  static constexpr int kSpecialToken = -1;
+  ExecutorVisionData() = default;
+  ExecutorVisionData(std::optional<TensorBuffer>&& embeddings, std::optional<TensorBuffer>&& per_layer_embeddings)
+      : embeddings_(std::move(embeddings)), per_layer_embeddings_(std::move(per_layer_embeddings)) {}
+  StatusOr<const TensorBuffer*> GetEmbeddingsPtr() const {
+    if (!embeddings_.has_value()) return NotFoundError("ExecutorVisionData::embeddings_ is not set.");
+    return &*embeddings_;
+  }
+  StatusOr<const TensorBuffer*> GetPerLayerEmbeddingsPtr() const {
+    if (!per_layer_embeddings_.has_value())
+      return NotFoundError("ExecutorVisionData::per_layer_embeddings_ is not set.");
+    return &*per_layer_embeddings_;
+  }
+
+ private:
+  std::optional<TensorBuffer> embeddings_;
+  std::optional<TensorBuffer> per_layer_embeddings_;
+};
+
 class ExecutorInputs {
  public:
   ExecutorInputs() = default;
   explicit ExecutorInputs(std::optional<ExecutorTextData> text) : text_data_(std::move(text)) {}
 
   StatusOr<const ExecutorTextData*> GetTextDataPtr() const {
-    if (!text_data_.has_value()) return FailedPreconditionError("ExecutorInputs::text_data_ is not set.");
+    if (!text_data_.has_value()) return NotFoundError("ExecutorInputs::text_data_ is not set.");
     return &*text_data_;
   }
   StatusOr<const TensorBuffer*> GetTextTokenIdsPtr() const {

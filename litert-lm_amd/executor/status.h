@@ -10,9 +10,13 @@
 #include <optional>
 #include <sstream>
 #include <string>
+#include <string_view>
 #include <utility>
 
 namespace litert::lm {
+
+// absl::string_view inside the reference tree (an alias of std::string_view in current abseil builds).
+using string_view = std::string_view;
 
 enum class StatusCode : int {
   kOk = 0,

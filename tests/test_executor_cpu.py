@@ -142,3 +142,25 @@ def test_fused_step_before_attention_keeps_the_step_logic():
             e.prefill([10, 11, 12, 13, 14, 15, 16])
             e.decode()
         assert ex.runs() == plain.runs() and ex.current_step() == plain.current_step() == 8
+
+
+def test_interface_matches_the_reference_header_method_for_method():
+    # names, return types, parameter types, constness and purity of every virtual method, in declaration order
+    import json
+    from cpp_interface import virtual_methods
+    with open(os.path.join(ROOT, "tests", "golden", "llm_executor_base_methods.json")) as f:
+        want = json.load(f)["methods"]
+    with open(os.path.join(ROOT, "litert-lm_amd", "executor", "llm_executor_base.h")) as f:
+        got = virtual_methods(f.read(), "LlmExecutorBase")
+    assert [m["name"] for m in want] == ["Prefill", "Prefill", "Decode", "Decode", "DecodeLogits", "ExecutorBackendName",
+                                         "GetVocabSize", "GetCurrentStep", "GetExecutorSettings", "FillVisionEmbeddings",
+                                         "Reset"]
+    assert got == want
+
+
+def test_vision_entry_point_keeps_the_base_class_default():
+    with make(runners=(4,)) as ex:
+        with pytest.raises(X.ExecutorError) as e:
+            ex.fill_vision_embeddings(0)
+        assert e.value.code == 12  # kUnimplemented
+        assert e.value.message == "FillVisionEmbeddings not implemented for backend: MI355X HIP attention"
