@@ -398,6 +398,19 @@ def pipeline_report(X, device_resident):
     return r["report"], float(pre.group(1)), float(dec.group(1))
 
 
+def protocol_layer_latency(A, torch, ctx=1152):
+    """Latency of one decode attention call (attention + merge launches, queued back to back) at the shape of the
+    benchmark protocol's decode turn: Hq4 / Hkv1, fp16, about the middle context of the 256 steps."""
+    at = A.Attn(1, 4, 1, D, 2048, 1, A.F16, A.F16)
+    fill_cache(at, torch, 1, [ctx], 1, torch.float16, seed=7)
+    q = torch.randn((1, 4, D), device="cuda:0", dtype=torch.float32).half()
+    out = torch.empty_like(q)
+    lens = A._i32_array([ctx])
+    sec, _ = time_steps(torch, lambda i: at.decode(0, lens, q, out, num_splits=0, batch=1), 500, 50)
+    at.close()
+    return sec
+
+
 def cpu_baseline_c3(layers, ctx, budget_s=24.0):
     """C restatement of the reference CPU op order (fp32, OpenMP) on the same
     30-layer decode sweep, repeated until about `budget_s` seconds are spent:
@@ -587,6 +600,12 @@ def main():
                 text, pre_tps, dec_tps = pipeline_report(X, resident)
                 log(f"[bench] the reference's benchmark protocol (1024 prefill / 256 decode ids), {mode}:\n" + text)
                 proto[mode] = {"prefill_tokens_per_s": pre_tps, "decode_tokens_per_s": dec_tps}
+            lat = protocol_layer_latency(A, torch)
+            proto["one_layer_decode_attention_latency_us"] = round(lat * 1e6, 2)
+            proto["decode_tokens_per_s_if_only_attention_ran"] = round(1.0 / (26 * lat), 1)
+            if "device_resident" in proto:
+                proto["device_resident_fraction_of_that"] = round(
+                    proto["device_resident"]["decode_tokens_per_s"] * 26 * lat, 3)
             result["pipeline_protocol"] = proto
 
     if not args.no_cpu:

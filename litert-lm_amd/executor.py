@@ -12,6 +12,8 @@ from . import attn as _attn
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhip_llm_executor.so")
 _lib = None
+# HipLlmExecutor(device_resident=True): activations, logits and sampling stay on the GPU for the whole pass.
+HAS_DEVICE_RESIDENT = True
 
 
 class ExecutorError(RuntimeError):
@@ -29,7 +31,7 @@ class _Config(ctypes.Structure):
         ("runner_lengths", ctypes.POINTER(ctypes.c_int32)),
         ("num_runners", ctypes.c_int32), ("fp16_activations", ctypes.c_int32),
         ("recording_backend", ctypes.c_int32), ("execute_pending_on_single_id_chunk", ctypes.c_int32),
-        ("softcap", ctypes.c_float), ("pre_attention", ctypes.c_int32),
+        ("softcap", ctypes.c_float), ("pre_attention", ctypes.c_int32), ("device_resident", ctypes.c_int32),
     ]
 
 
@@ -52,6 +54,9 @@ def lib():
         L.hle_destroy.argtypes = [vp]
         L.hle_destroy.restype = None
         L.hle_prefill.argtypes = [vp, i32p, i32, i32, errp]
+        L.hle_prefill_with_params.argtypes = [vp, i32p, i32, i32, i32, i32, errp]
+        L.hle_is_device_resident.argtypes = [vp]
+        L.hle_wait_for_completion.argtypes = [vp, errp]
         L.hle_decode.argtypes = [vp, i32p, errp]
         L.hle_decode_logits.argtypes = [vp, i32, ctypes.POINTER(ctypes.c_float), errp]
         for n in ("hle_current_step", "hle_vocab_size", "hle_max_num_tokens", "hle_num_runs"):
@@ -105,13 +110,16 @@ class HipLlmExecutor:
 
     def __init__(self, num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens, runner_lengths=(1024,),
                  layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=False,
-                 softcap=0.0, pre_attention=False):
+                 softcap=0.0, pre_attention=False, device_resident=None):
+        """device_resident: True / False, or None to let the executor decide (device-resident on its own MI355X
+        backend, host-staged on the recording backend)."""
         self._win = _arr(layer_window) if layer_window is not None else None
         self._runners = _arr(runner_lengths)
         cfg = _Config(num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens,
                       ctypes.cast(self._win, ctypes.POINTER(ctypes.c_int32)) if self._win is not None else None,
                       ctypes.cast(self._runners, ctypes.POINTER(ctypes.c_int32)), len(runner_lengths), int(fp16),
-                      int(recording_backend), int(execute_pending_on_single_id_chunk), softcap, int(pre_attention))
+                      int(recording_backend), int(execute_pending_on_single_id_chunk), softcap, int(pre_attention),
+                      -1 if device_resident is None else int(bool(device_resident)))
         self._h = ctypes.c_void_p()
         err = ctypes.c_void_p()
         _check(lib().hle_create(ctypes.byref(cfg), ctypes.byref(self._h), ctypes.byref(err)), err)
@@ -134,11 +142,24 @@ class HipLlmExecutor:
     def __exit__(self, *exc):
         self.close()
 
-    def prefill(self, ids, batch=1):
+    def prefill(self, ids, batch=1, wait_for_completion=None, cancel=None):
+        """Prefill(inputs), or Prefill(inputs, params) when wait_for_completion or cancel (the value the cancel
+        flag holds during the call) is given."""
         ids = list(ids)
         n = len(ids) // batch if batch else 0
         err = ctypes.c_void_p()
-        _check(lib().hle_prefill(self._h, _arr(ids), batch, n, ctypes.byref(err)), err)
+        if wait_for_completion is None and cancel is None:
+            _check(lib().hle_prefill(self._h, _arr(ids), batch, n, ctypes.byref(err)), err)
+        else:
+            _check(lib().hle_prefill_with_params(self._h, _arr(ids), batch, n, int(bool(wait_for_completion)),
+                                                 -1 if cancel is None else int(bool(cancel)), ctypes.byref(err)), err)
+
+    def is_device_resident(self) -> bool:
+        return bool(lib().hle_is_device_resident(self._h))
+
+    def wait_for_completion(self):
+        err = ctypes.c_void_p()
+        _check(lib().hle_wait_for_completion(self._h, ctypes.byref(err)), err)
 
     def decode(self) -> int:
         tok = ctypes.c_int32(-7)

@@ -56,6 +56,24 @@ class AttentionBackend {
   virtual Status Decode(int layer, int kv_len, const float* q, float* out) = 0;
   virtual Status Reset() = 0;
   virtual std::string Name() const = 0;
+
+  // Device-resident form: the rows are device buffers in the activation type of the backend (float32, or IEEE half
+  // for fp16 activations), every call is queued on Stream() and returns without waiting, results are ordered by the
+  // stream. This is how the reference's GPU branch runs: cache and activations stay in device buffers across
+  // signatures (llm_litert_compiled_model_executor.cc:753-755). A backend is either host-staged (the calls above) or
+  // device-resident (the calls below); the other set answers kFailedPrecondition.
+  virtual bool DeviceResident() const { return false; }
+  virtual void* Stream() const { return nullptr; }  // hipStream_t
+  virtual Status AppendOnDevice(int, int, int, const void*, const void*) { return NotDeviceResident(); }
+  virtual Status PreAttentionOnDevice(int, int, int, void*, const void*, const void*) { return NotDeviceResident(); }
+  virtual Status PrefillOnDevice(int, int, int, const void*, void*) { return NotDeviceResident(); }
+  virtual Status DecodeOnDevice(int, int, const void*, void*) { return NotDeviceResident(); }
+  virtual Status Sync() { return OkStatus(); }  // waits for everything queued on Stream()
+
+ protected:
+  Status NotDeviceResident() const {
+    return FailedPreconditionError("attention backend '" + Name() + "' is not device-resident.");
+  }
 };
 
 struct AttentionCall {
@@ -98,10 +116,10 @@ class RecordingAttentionBackend : public AttentionBackend {
   AttentionShape shape_;
 };
 
-// fp32 activations: fp32 cache and I/O. fp16 activations: fp16 cache and I/O
-// (converted on the host at this boundary).
+// fp32 activations: fp32 cache and I/O. fp16 activations: fp16 cache and I/O (converted on the host at this
+// boundary when host-staged). device_resident: the handle takes device pointers and runs on a stream of its own.
 StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const AttentionShape& shape, bool fp16,
-                                                                         int device);
+                                                                         int device, bool device_resident = false);
 
 }  // namespace litert::lm
 #endif  // LITERT_LM_AMD_EXECUTOR_ATTENTION_BACKEND_H_

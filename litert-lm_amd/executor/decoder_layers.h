@@ -33,6 +33,36 @@ class DecoderLayers {
   virtual Status ConsumeAttention(int layer, const float* attn) = 0;
   // Logits [vocab] of the last token of this pass.
   virtual Status Logits(float* logits) = 0;
+
+  // Device-resident form of the same pass. The buffers are device memory in the activation type of the executor
+  // (`fp16`: IEEE half, else float32), sized for `n` tokens; all work is queued on `stream` (a hipStream_t) and no
+  // call waits. The graph between two attention ops is one segment: what follows attention of layer l (output
+  // projection, MLP, norms) and what precedes attention of layer l + 1 (its q / k / v projections).
+  struct DeviceActivations {
+    void* q = nullptr;     // [n][Hq][D]
+    void* k = nullptr;     // [n][Hkv][D]
+    void* v = nullptr;     // [n][Hkv][D]
+    void* attn = nullptr;  // [n][Hq][D]
+    bool fp16 = false;
+    void* stream = nullptr;
+  };
+  virtual bool HasDeviceForm() const { return false; }
+  // Starts a pass (tokens and positions are host arrays, consumed before the call returns) and fills q / k / v of layer 0.
+  virtual Status BeginOnDevice(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions,
+                               const DeviceActivations& io) {
+    (void)tokens, (void)positions, (void)io;
+    return UnimplementedError("these decoder layers have no device-resident form.");
+  }
+  // Consumes io.attn of `layer` and, unless it was the last layer, fills q / k / v of layer + 1.
+  virtual Status NextLayerOnDevice(int layer, const DeviceActivations& io) {
+    (void)layer, (void)io;
+    return UnimplementedError("these decoder layers have no device-resident form.");
+  }
+  // Logits [vocab] float32 (device memory) of the last token of this pass.
+  virtual Status LogitsOnDevice(float* logits, void* stream) {
+    (void)logits, (void)stream;
+    return UnimplementedError("these decoder layers have no device-resident form.");
+  }
 };
 
 class SyntheticDecoderLayers : public DecoderLayers {
@@ -44,6 +74,14 @@ class SyntheticDecoderLayers : public DecoderLayers {
   Status ProjectQkv(int layer, float* q, float* k, float* v) override;
   Status ConsumeAttention(int layer, const float* attn) override;
   Status Logits(float* logits) override;
+
+  // The same arithmetic as kernels (synthetic_decoder_layers_device.hip).
+  ~SyntheticDecoderLayers() override;
+  bool HasDeviceForm() const override { return true; }
+  Status BeginOnDevice(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions,
+                       const DeviceActivations& io) override;
+  Status NextLayerOnDevice(int layer, const DeviceActivations& io) override;
+  Status LogitsOnDevice(float* logits, void* stream) override;
 
   // Deterministic norm weights and rotary frequencies in the pattern of Gemma 3
   // (query / key norm with a (1 + weight) scale, theta 10,000 on windowed layers
@@ -67,6 +105,16 @@ class SyntheticDecoderLayers : public DecoderLayers {
   int vocab_;
   int n_ = 0;
   std::vector<float> state_;  // [n][hidden]
+  // device-resident pass: state [capacity][hidden] float32 and the token ids of a long pass, in device memory
+  float* d_state_ = nullptr;
+  int32_t* d_tokens_ = nullptr;
+  int d_capacity_ = 0;
+  int d_n_ = 0;
+  // pinned host slots the ids of long passes are copied from, each with the event that says its copy has run
+  static constexpr int kTokenStages = 4;
+  int32_t* stage_ids_[kTokenStages] = {};
+  void* stage_done_[kTokenStages] = {};  // hipEvent_t
+  int stage_next_ = 0;
 };
 
 }  // namespace litert::lm

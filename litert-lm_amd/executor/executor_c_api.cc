@@ -2,6 +2,7 @@
 // executor over the synthetic decoder layers, drive Prefill / Decode, read the
 // trace of forward passes. Status codes are absl::StatusCode integers; error
 // text is malloc'd for the caller to free().
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
@@ -47,6 +48,7 @@ struct hle_config {
   int32_t execute_pending_on_single_id_chunk;
   float softcap;
   int32_t pre_attention;             // 1: the layers hand over raw projections; Gemma-3-like norm + rotary constants
+  int32_t device_resident;           // -1: the executor decides, 0: host-staged, 1: device-resident
 };
 
 int hle_create(const hle_config* c, void** out, char** err) {
@@ -67,6 +69,9 @@ int hle_create(const hle_config* c, void** out, char** err) {
   HipExecutorOptions options;
   options.prefill_runner_lengths.assign(c->runner_lengths, c->runner_lengths + c->num_runners);
   options.execute_pending_on_single_id_chunk = c->execute_pending_on_single_id_chunk != 0;
+  options.residency = c->device_resident < 0    ? HipExecutorOptions::Residency::kAuto
+                      : c->device_resident == 0 ? HipExecutorOptions::Residency::kHost
+                                                : HipExecutorOptions::Residency::kDevice;
   std::unique_ptr<AttentionBackend> backend;
   if (c->recording_backend) backend = std::make_unique<RecordingAttentionBackend>(shape);
   auto ex = HipLlmExecutor::Create(*settings, std::make_unique<SyntheticDecoderLayers>(shape, c->vocab), options,
@@ -80,6 +85,18 @@ void hle_destroy(void* h) { delete static_cast<HipLlmExecutor*>(h); }
 
 int hle_prefill(void* h, const int32_t* ids, int32_t batch, int32_t n, char** err) {
   return Finish(static_cast<HipLlmExecutor*>(h)->Prefill(IdsInput(ids, batch, n)), err);
+}
+
+// Prefill with parameters: `cancel` is the value the caller's cancel flag holds during the call (-1: no flag).
+int hle_prefill_with_params(void* h, const int32_t* ids, int32_t batch, int32_t n, int32_t wait_for_completion,
+                            int32_t cancel, char** err) {
+  std::atomic_bool flag(cancel > 0);
+  ExecutorPrefillParams params(-1, wait_for_completion != 0, cancel < 0 ? nullptr : &flag);
+  return Finish(static_cast<HipLlmExecutor*>(h)->Prefill(IdsInput(ids, batch, n), params), err);
+}
+int hle_is_device_resident(void* h) { return static_cast<HipLlmExecutor*>(h)->device_resident() ? 1 : 0; }
+int hle_wait_for_completion(void* h, char** err) {
+  return Finish(static_cast<HipLlmExecutor*>(h)->WaitForCompletion(), err);
 }
 
 int hle_decode(void* h, int32_t* out_token, char** err) {

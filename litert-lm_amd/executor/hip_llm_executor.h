@@ -32,6 +32,14 @@ struct HipExecutorOptions {
   // pending token first (opt-in fix: GetCurrentStep then reads one higher than
   // the reference's after such a call).
   bool execute_pending_on_single_id_chunk = false;
+  // Where activations live. kDevice: q / k / v / attention output, logits and the sampled id stay in device memory
+  // for the whole forward pass, every layer is queued on the attention backend's stream without a wait in between,
+  // Decode(tokens) samples on the device (libmi355_sampler.so) and only the id comes back; Prefill returns after
+  // queueing unless the prefill parameters ask to wait. This is the reference's GPU arrangement
+  // (llm_litert_compiled_model_executor.cc:536-566,753-755). kHost: float32 host rows staged through the boundary
+  // per call. kAuto: kDevice when the decoder layers have a device form and no backend was injected, else kHost.
+  enum class Residency { kAuto, kHost, kDevice };
+  Residency residency = Residency::kAuto;
 };
 
 // One forward pass as the executor issued it (kept for tests and debugging).
@@ -63,8 +71,12 @@ class HipLlmExecutor : public LlmExecutorBase {
   StatusOr<LlmExecutorSettings> GetExecutorSettings() const override { return settings_; }
   Status Reset() override;
 
+  ~HipLlmExecutor() override;
   const std::vector<ExecutorRunRecord>& run_records() const { return records_; }
   AttentionBackend* attention_backend() { return backend_.get(); }
+  bool device_resident() const { return device_ != nullptr; }
+  // Waits for everything this executor has queued (a no-op when host-staged).
+  Status WaitForCompletion();
 
  private:
   HipLlmExecutor(LlmExecutorSettings settings, std::unique_ptr<DecoderLayers> layers, HipExecutorOptions options,
@@ -76,6 +88,12 @@ class HipLlmExecutor : public LlmExecutorBase {
   // cache row of the first one); logits of the last token if asked for.
   Status RunTokens(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions, bool is_decode,
                    bool want_logits);
+  Status RunTokensOnDevice(const std::vector<int32_t>& tokens, const std::vector<int32_t>& positions, bool is_decode,
+                           bool want_logits);
+  // Device-resident decode step: logits stay in device memory (copied to logits_ only when `fetch_logits`).
+  Status FetchLogits();
+  struct DeviceState;  // device buffers, sampler handle, pinned id slot
+  Status InitDeviceState();
 
   LlmExecutorSettings settings_;
   std::unique_ptr<DecoderLayers> layers_;
@@ -87,6 +105,7 @@ class HipLlmExecutor : public LlmExecutorBase {
   TensorBuffer logits_;  // [1, 1, vocab] float32
   std::vector<float> q_, k_, v_, attn_;
   std::vector<ExecutorRunRecord> records_;
+  std::unique_ptr<DeviceState> device_;  // null: host-staged
 };
 
 }  // namespace litert::lm

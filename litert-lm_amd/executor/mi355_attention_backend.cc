@@ -1,9 +1,11 @@
-// AttentionBackend over the C ABI of libmi355_attn.so. Host float32 rows cross
-// the boundary as they are (fp32 cache) or as fp16 (fp16 cache); the library
-// stages them to the device (host_io = 1) and returns with results in place,
-// which is what the executor's synchronous Decode contract needs
-// (runtime/executor/llm_litert_compiled_model_executor.cc:528-533 hands out a
-// host-visible logits buffer right after the step).
+// AttentionBackend over the C ABI of libmi355_attn.so, in one of two forms.
+// Host-staged: host float32 rows cross the boundary as they are (fp32 cache) or
+// as fp16 (fp16 cache); the library stages them to the device (host_io = 1) and
+// returns with results in place. Device-resident: the handle takes device
+// pointers (host_io = 0) and queues every call on its own stream without
+// waiting, so a forward pass over all layers runs without a host round trip,
+// as the reference's GPU branch does with its device-side cache and activation
+// buffers (runtime/executor/llm_litert_compiled_model_executor.cc:753-755).
 #include <cstdlib>
 #include <string>
 #include <vector>
@@ -23,10 +25,40 @@ Status FromCode(int rc, char* err, const char* what) {
 
 class Mi355AttentionBackend : public AttentionBackend {
  public:
-  Mi355AttentionBackend(mi355_attn* h, AttentionShape shape, bool fp16) : h_(h), shape_(std::move(shape)), fp16_(fp16) {}
+  Mi355AttentionBackend(mi355_attn* h, AttentionShape shape, bool fp16, bool device_resident)
+      : h_(h), shape_(std::move(shape)), fp16_(fp16), device_resident_(device_resident) {}
   ~Mi355AttentionBackend() override { mi355_attn_destroy(h_); }
 
+  bool DeviceResident() const override { return device_resident_; }
+  void* Stream() const override { return mi355_attn_stream(h_); }
+  Status AppendOnDevice(int layer, int pos, int n, const void* k, const void* v) override {
+    if (!device_resident_) return NotDeviceResident();
+    char* err = nullptr;
+    return FromCode(mi355_attn_kv_append(h_, layer, 0, pos, n, k, v, &err), err, "kv_append");
+  }
+  Status PreAttentionOnDevice(int layer, int pos, int n, void* q, const void* k, const void* v) override {
+    if (!device_resident_) return NotDeviceResident();
+    char* err = nullptr;
+    return FromCode(mi355_attn_pre_attention(h_, layer, 0, pos, n, q, k, v, q, &err), err, "pre_attention");
+  }
+  Status PrefillOnDevice(int layer, int q_pos0, int n, const void* q, void* out) override {
+    if (!device_resident_) return NotDeviceResident();
+    char* err = nullptr;
+    return FromCode(mi355_attn_prefill(h_, layer, 0, q_pos0, n, q, out, &err), err, "prefill");
+  }
+  Status DecodeOnDevice(int layer, int kv_len, const void* q, void* out) override {
+    if (!device_resident_) return NotDeviceResident();
+    char* err = nullptr;
+    const int32_t len = kv_len;
+    return FromCode(mi355_attn_decode(h_, layer, nullptr, &len, 1, q, out, 0, &err), err, "decode");
+  }
+  Status Sync() override {
+    char* err = nullptr;
+    return FromCode(mi355_attn_sync(h_, &err), err, "sync");
+  }
+
   Status Append(int layer, int pos, int n, const float* k, const float* v) override {
+    if (device_resident_) return HostStagedOnly();
     char* err = nullptr;
     const size_t count = (size_t)n * shape_.num_kv_heads * shape_.head_dim;
     int rc;
@@ -41,6 +73,7 @@ class Mi355AttentionBackend : public AttentionBackend {
   }
 
   Status PreAttention(int layer, int pos, int n, float* q, const float* k, const float* v) override {
+    if (device_resident_) return HostStagedOnly();
     char* err = nullptr;
     const size_t qn = (size_t)n * shape_.num_q_heads * shape_.head_dim;
     const size_t kn = (size_t)n * shape_.num_kv_heads * shape_.head_dim;
@@ -58,6 +91,7 @@ class Mi355AttentionBackend : public AttentionBackend {
   }
 
   Status Prefill(int layer, int q_pos0, int n, const float* q, float* out) override {
+    if (device_resident_) return HostStagedOnly();
     char* err = nullptr;
     const size_t count = (size_t)n * shape_.num_q_heads * shape_.head_dim;
     int rc;
@@ -73,6 +107,7 @@ class Mi355AttentionBackend : public AttentionBackend {
   }
 
   Status Decode(int layer, int kv_len, const float* q, float* out) override {
+    if (device_resident_) return HostStagedOnly();
     char* err = nullptr;
     const size_t count = (size_t)shape_.num_q_heads * shape_.head_dim;
     const int32_t len = kv_len;
@@ -96,6 +131,9 @@ class Mi355AttentionBackend : public AttentionBackend {
   std::string Name() const override { return mi355_attn_version(); }
 
  private:
+  Status HostStagedOnly() const {
+    return FailedPreconditionError("this attention backend is device-resident: it takes device buffers.");
+  }
   static void ToHalf(const float* src, size_t n, std::vector<_Float16>* dst) {
     dst->resize(n);
     for (size_t i = 0; i < n; ++i) (*dst)[i] = static_cast<_Float16>(src[i]);
@@ -106,13 +144,14 @@ class Mi355AttentionBackend : public AttentionBackend {
   mi355_attn* h_;
   AttentionShape shape_;
   bool fp16_;
+  bool device_resident_;
   std::vector<_Float16> ha_, hb_, hq_;
 };
 
 }  // namespace
 
 StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const AttentionShape& shape, bool fp16,
-                                                                         int device) {
+                                                                         int device, bool device_resident) {
   mi355_attn_config cfg{};
   cfg.struct_size = sizeof(cfg);
   cfg.num_layers = shape.num_layers;
@@ -127,7 +166,7 @@ StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const At
   cfg.softcap = shape.softcap;
   cfg.layer_window = shape.layer_window.empty() ? nullptr : shape.layer_window.data();
   cfg.device = device;
-  cfg.host_io = 1;
+  cfg.host_io = device_resident ? 0 : 1;
   cfg.own_stream = 1;
   mi355_attn* h = nullptr;
   char* err = nullptr;
@@ -161,7 +200,7 @@ StatusOr<std::unique_ptr<AttentionBackend>> CreateMi355AttentionBackend(const At
       return FromCode(trc, err, "mi355_attn_set_layer_transform");
     }
   }
-  return std::unique_ptr<AttentionBackend>(new Mi355AttentionBackend(h, shape, fp16));
+  return std::unique_ptr<AttentionBackend>(new Mi355AttentionBackend(h, shape, fp16, device_resident));
 }
 
 }  // namespace litert::lm

@@ -20,6 +20,7 @@ using string_view = std::string_view;
 
 enum class StatusCode : int {
   kOk = 0,
+  kCancelled = 1,
   kInvalidArgument = 3,
   kNotFound = 5,
   kAlreadyExists = 6,
@@ -45,6 +46,7 @@ class Status {
 };
 
 inline Status OkStatus() { return Status(); }
+inline Status CancelledError(std::string m) { return Status(StatusCode::kCancelled, std::move(m)); }
 inline Status InvalidArgumentError(std::string m) { return Status(StatusCode::kInvalidArgument, std::move(m)); }
 inline Status InternalError(std::string m) { return Status(StatusCode::kInternal, std::move(m)); }
 inline Status UnimplementedError(std::string m) { return Status(StatusCode::kUnimplemented, std::move(m)); }
@@ -52,6 +54,8 @@ inline Status FailedPreconditionError(std::string m) { return Status(StatusCode:
 inline Status AlreadyExistsError(std::string m) { return Status(StatusCode::kAlreadyExists, std::move(m)); }
 inline Status NotFoundError(std::string m) { return Status(StatusCode::kNotFound, std::move(m)); }
 inline Status OutOfRangeError(std::string m) { return Status(StatusCode::kOutOfRange, std::move(m)); }
+inline Status UnavailableError(std::string m) { return Status(StatusCode::kUnavailable, std::move(m)); }
+inline Status ResourceExhaustedError(std::string m) { return Status(StatusCode::kResourceExhausted, std::move(m)); }
 
 template <class T>
 class StatusOr {

@@ -164,3 +164,21 @@ def test_vision_entry_point_keeps_the_base_class_default():
             ex.fill_vision_embeddings(0)
         assert e.value.code == 12  # kUnimplemented
         assert e.value.message == "FillVisionEmbeddings not implemented for backend: MI355X HIP attention"
+
+
+def test_prefill_params_cancel_and_wait():
+    with make(runners=(4,)) as ex:
+        assert not ex.is_device_resident()          # the recording backend is host-staged
+        with pytest.raises(X.ExecutorError) as e:
+            ex.prefill([1, 2, 3, 4, 5, 6], cancel=True)
+        assert e.value.code == 1 and "cancelled" in e.value.message   # kCancelled before the first chunk
+        assert ex.runs() == [] and ex.current_step() == 0
+        ex.prefill([1, 2, 3, 4, 5, 6], wait_for_completion=True, cancel=False)
+        assert ex.current_step() == 6 and len(ex.runs()) == 2
+        ex.wait_for_completion()                    # nothing is ever pending on a host-staged executor
+
+
+def test_device_resident_needs_a_device_resident_backend():
+    with pytest.raises(X.ExecutorError) as e:
+        make(device_resident=True)
+    assert e.value.code == INVALID_ARGUMENT and "device-resident" in e.value.message
