@@ -62,115 +62,142 @@ std::string FormatDuration(Duration d) {
   return s;
 }
 
-Status BenchmarkInfo::TimeInitPhaseStart(const std::string& phase_name) {
-  if (start_time_map_.count(phase_name)) return InternalError("Phase " + phase_name + " already started.");
-  start_time_map_[phase_name] = Now();
+namespace {
+struct SectionWords {
+  const char* noun;         // in the error texts
+  const char* label_stem;   // of a turn label, null for named rows
+};
+const SectionWords& Words(BenchmarkInfo::Section s) {
+  static const SectionWords kWords[] = {{"Phase", nullptr}, {"Prefill turn", "prefill:"}, {"Decode turn", "decode:"},
+                                        {"Mark", nullptr}};
+  return kWords[static_cast<int>(s)];
+}
+}  // namespace
+
+std::string BenchmarkInfo::TurnLabel(Section section) const {
+  return Words(section).label_stem + std::to_string(Count(section));
+}
+
+BenchmarkInfo::Row* BenchmarkInfo::Find(Section section, const std::string& label) {
+  const bool mark = section == Section::kMark;
+  for (Row& row : rows_)
+    if ((row.section == Section::kMark) == mark && row.label == label) return &row;
+  return nullptr;
+}
+
+Status BenchmarkInfo::Start(Section section, const std::string& label) {
+  if (Find(section, label) != nullptr)
+    return InternalError(std::string(Words(section).noun) + " " + label + " already started.");
+  rows_.push_back(Row{section, label, Now()});
   return OkStatus();
 }
 
-Status BenchmarkInfo::TimeInitPhaseEnd(const std::string& phase_name) {
-  if (!start_time_map_.count(phase_name)) return InternalError("Phase " + phase_name + " not started.");
-  init_phases_[phase_name] = std::chrono::duration_cast<Duration>(Now() - start_time_map_[phase_name]);
+Status BenchmarkInfo::Stop(Section section, const std::string& label, uint64_t tokens) {
+  const TimePoint now = Now();
+  Row* row = Find(section, label);
+  if (row == nullptr) return InternalError(std::string(Words(section).noun) + " " + label + " not started.");
+  // A phase may be ended again: the later reading replaces the earlier one. The row counts for the section that
+  // ends it (which only differs from the one that started it when a phase was named like a turn).
+  row->section = section;
+  row->took = std::chrono::duration_cast<Duration>(now - row->since);
+  row->tokens = tokens;
+  row->measured = true;
   return OkStatus();
 }
 
 Status BenchmarkInfo::TimeMarkDelta(const std::string& mark_name) {
   const TimePoint now = Now();
-  auto it = mark_time_map_.find(mark_name);
-  if (it != mark_time_map_.end()) mark_durations_[mark_name] = std::chrono::duration_cast<Duration>(now - it->second);
-  mark_time_map_[mark_name] = now;
+  if (Row* row = Find(Section::kMark, mark_name)) {
+    row->took = std::chrono::duration_cast<Duration>(now - row->since);
+    row->measured = true;
+    row->since = now;
+  } else {
+    rows_.push_back(Row{Section::kMark, mark_name, now});
+  }
   return OkStatus();
 }
 
-Status BenchmarkInfo::TimePrefillTurnStart() {
-  const std::string phase_name = "prefill:" + std::to_string(prefill_turn_index_);
-  if (start_time_map_.count(phase_name)) return InternalError("Prefill turn " + phase_name + " already started.");
-  start_time_map_[phase_name] = Now();
-  return OkStatus();
+std::map<std::string, Duration> BenchmarkInfo::Named(Section section) const {
+  std::map<std::string, Duration> out;
+  for (const Row& row : rows_)
+    if (row.section == section && row.measured) out[row.label] = row.took;
+  return out;
 }
 
-Status BenchmarkInfo::TimePrefillTurnEnd(uint64_t num_prefill_tokens) {
-  const std::string phase_name = "prefill:" + std::to_string(prefill_turn_index_);
-  if (!start_time_map_.count(phase_name)) return InternalError("Prefill turn " + phase_name + " not started.");
-  prefill_turns_.emplace_back(num_prefill_tokens, std::chrono::duration_cast<Duration>(Now() - start_time_map_[phase_name]));
-  prefill_turn_index_++;
-  return OkStatus();
+uint64_t BenchmarkInfo::Count(Section section) const {
+  uint64_t n = 0;
+  for (const Row& row : rows_) n += row.section == section && row.measured;
+  return n;
 }
 
-Status BenchmarkInfo::TimeDecodeTurnStart() {
-  const std::string phase_name = "decode:" + std::to_string(decode_turn_index_);
-  if (start_time_map_.count(phase_name)) return InternalError("Decode turn " + phase_name + " already started.");
-  start_time_map_[phase_name] = Now();
-  return OkStatus();
+const BenchmarkInfo::Row* BenchmarkInfo::TurnRow(Section section, int turn_index) const {
+  if (turn_index < 0) return nullptr;
+  for (const Row& row : rows_)
+    if (row.section == section && row.measured && turn_index-- == 0) return &row;
+  return nullptr;
 }
 
-Status BenchmarkInfo::TimeDecodeTurnEnd(uint64_t num_decode_tokens) {
-  const std::string phase_name = "decode:" + std::to_string(decode_turn_index_);
-  if (!start_time_map_.count(phase_name)) return InternalError("Decode turn " + phase_name + " not started.");
-  decode_turns_.emplace_back(num_decode_tokens, std::chrono::duration_cast<Duration>(Now() - start_time_map_[phase_name]));
-  decode_turn_index_++;
-  return OkStatus();
+BenchmarkTurnData BenchmarkInfo::Turn(Section section, int turn_index) const {
+  const Row* row = TurnRow(section, turn_index);
+  return row ? BenchmarkTurnData(row->tokens, row->took) : BenchmarkTurnData(0, Duration::zero());
 }
 
-double BenchmarkInfo::TokensPerSec(const std::vector<BenchmarkTurnData>& turns, int turn_index) {
-  if (turn_index < 0 || static_cast<size_t>(turn_index) >= turns.size()) return 0.0;
-  const BenchmarkTurnData& turn = turns[turn_index];
-  if (turn.duration <= Duration::zero()) return 0.0;
-  const double seconds = static_cast<double>(turn.duration.count()) * 1e-9;
-  if (seconds <= 0.0) return 0.0;
-  return static_cast<double>(turn.num_tokens) / seconds;
+double BenchmarkInfo::TokensPerSec(Section section, int turn_index) const {
+  const Row* row = TurnRow(section, turn_index);
+  if (row == nullptr || row->took <= Duration::zero()) return 0.0;
+  const double seconds = static_cast<double>(row->took.count()) * 1e-9;
+  return seconds > 0.0 ? static_cast<double>(row->tokens) / seconds : 0.0;
 }
-
-double BenchmarkInfo::GetPrefillTokensPerSec(int turn_index) const { return TokensPerSec(prefill_turns_, turn_index); }
-double BenchmarkInfo::GetDecodeTokensPerSec(int turn_index) const { return TokensPerSec(decode_turns_, turn_index); }
 
 std::ostream& operator<<(std::ostream& os, const BenchmarkTurnData& data) {
-  os << "Processed " << data.num_tokens << " tokens in " << FormatDuration(data.duration) << " duration." << std::endl;
-  return os;
+  return os << "Processed " << data.num_tokens << " tokens in " << FormatDuration(data.duration) << " duration.\n"
+            << std::flush;
 }
 
+// The report, section by section, in the reference's wording (io_types.cc:255-308): two decimals throughout,
+// a rule after every section, the marks only when there are any.
 std::ostream& operator<<(std::ostream& os, const BenchmarkInfo& info) {
-  os << std::fixed << std::setprecision(2);
-  os << "BenchmarkInfo:" << std::endl;
-  os << "  Init Phases (" << info.GetInitPhases().size() << "):" << std::endl;
-  if (info.GetInitPhases().empty()) {
-    os << "    No init phases recorded." << std::endl;
-  } else {
-    double total_time = 0.0;
-    for (const auto& phase : info.GetInitPhases()) {
-      total_time += Millis(phase.second);
-      os << "    - " << phase.first << ": " << Millis(phase.second) << " ms" << std::endl;
+  static const char kRule[] = "--------------------------------------------------\n";
+  os << std::fixed << std::setprecision(2) << "BenchmarkInfo:\n";
+
+  const auto phases = info.GetInitPhases();
+  os << "  Init Phases (" << phases.size() << "):\n";
+  double total_ms = 0.0;
+  for (const auto& [name, took] : phases) {
+    total_ms += Millis(took);
+    os << "    - " << name << ": " << Millis(took) << " ms\n";
+  }
+  if (phases.empty()) os << "    No init phases recorded.\n";
+  else os << "    Total init time: " << total_ms << " ms\n";
+  os << kRule;
+
+  struct TurnSection {
+    const char* title;
+    const char* lower;
+    uint64_t turns;
+    BenchmarkTurnData (BenchmarkInfo::*turn)(int) const;
+    double (BenchmarkInfo::*speed)(int) const;
+  };
+  const TurnSection sections[] = {
+      {"Prefill", "prefill", info.GetTotalPrefillTurns(), &BenchmarkInfo::GetPrefillTurn,
+       &BenchmarkInfo::GetPrefillTokensPerSec},
+      {"Decode", "decode", info.GetTotalDecodeTurns(), &BenchmarkInfo::GetDecodeTurn,
+       &BenchmarkInfo::GetDecodeTokensPerSec}};
+  for (const TurnSection& s : sections) {
+    os << "  " << s.title << " Turns (Total: " << s.turns << "):\n";
+    if (s.turns == 0) os << "    No " << s.lower << " turns recorded.\n";
+    for (uint64_t i = 0; i < s.turns; ++i) {
+      const int turn = static_cast<int>(i);
+      os << "    " << s.title << " Turn " << i + 1 << ": " << (info.*s.turn)(turn);
+      os << "      " << s.title << " Speed: " << (info.*s.speed)(turn) << " tokens/sec.\n";
     }
-    os << "    Total init time: " << total_time << " ms" << std::endl;
+    os << kRule;
   }
-  os << "--------------------------------------------------" << std::endl;
-  os << "  Prefill Turns (Total: " << info.GetTotalPrefillTurns() << "):" << std::endl;
-  if (info.GetTotalPrefillTurns() == 0) {
-    os << "    No prefill turns recorded." << std::endl;
-  } else {
-    for (uint64_t i = 0; i < info.GetTotalPrefillTurns(); ++i) {
-      os << "    Prefill Turn " << i + 1 << ": " << info.GetPrefillTurn(static_cast<int>(i));
-      os << "      Prefill Speed: " << info.GetPrefillTokensPerSec(static_cast<int>(i)) << " tokens/sec." << std::endl;
-    }
-  }
-  os << "--------------------------------------------------" << std::endl;
-  os << "  Decode Turns (Total: " << info.GetTotalDecodeTurns() << "):" << std::endl;
-  if (info.GetTotalDecodeTurns() == 0) {
-    os << "    No decode turns recorded." << std::endl;
-  } else {
-    for (uint64_t i = 0; i < info.GetTotalDecodeTurns(); ++i) {
-      os << "    Decode Turn " << i + 1 << ": " << info.GetDecodeTurn(static_cast<int>(i));
-      os << "      Decode Speed: " << info.GetDecodeTokensPerSec(static_cast<int>(i)) << " tokens/sec." << std::endl;
-    }
-  }
-  os << "--------------------------------------------------" << std::endl;
-  if (!info.GetMarkDurations().empty()) {
-    os << "  Mark Durations (" << info.GetMarkDurations().size() << "):" << std::endl;
-    for (const auto& mark : info.GetMarkDurations())
-      os << "    - " << mark.first << ": " << FormatDuration(mark.second) << std::endl;
-  }
-  os << "--------------------------------------------------" << std::endl;
-  return os;
+
+  const auto marks = info.GetMarkDurations();
+  if (!marks.empty()) os << "  Mark Durations (" << marks.size() << "):\n";
+  for (const auto& [name, took] : marks) os << "    - " << name << ": " << FormatDuration(took) << "\n";
+  return os << kRule << std::flush;
 }
 
 }  // namespace litert::lm

@@ -6,108 +6,105 @@
 namespace litert::lm {
 namespace {
 
-constexpr int kDefaultMaxNumTokens = 4096;  // when the executor has no settings to ask (pipeline.cc:50-62)
+// Why a decode loop ends (runtime/core/pipeline.cc:64-84), in the order the conditions are tried.
+enum class LoopEnd { kGoOn, kStopTokens, kStepBudget, kCacheFull };
 
-int TryGetMaxNumTokens(const LlmExecutor& executor) {
-  auto settings = executor.GetExecutorSettings();
-  return settings.ok() ? settings->GetMaxNumTokens() : kDefaultMaxNumTokens;
-}
-
-// (true, cache_full): the loop ends; cache_full tells why.
-std::pair<bool, bool> ShouldStop(bool hit_stop_tokens, int benchmark_decode_token_count, int num_decoded_steps,
-                                 int current_step, int max_num_tokens) {
-  if (hit_stop_tokens && benchmark_decode_token_count == 0) return {true, false};
-  if (benchmark_decode_token_count > 0 && num_decoded_steps >= benchmark_decode_token_count) return {true, false};
-  if (current_step >= max_num_tokens) return {true, true};
-  return {false, false};
-}
-
-// One decode step with sampling inside the executor (pipeline.cc:160-227).
-class DecodeInternalSamplingOneStep {
- public:
-  DecodeInternalSamplingOneStep(LlmExecutor& executor, const StopTokenDetector& detector,
-                                std::optional<BenchmarkInfo>& benchmark_info)
-      : executor_(executor), benchmark_info_(benchmark_info), detector_(detector) {
-    output_tokens_ = TensorBuffer::Create(ElementType::kInt32, {1, 1});
-  }
-  StatusOr<bool> Run() {
-    if (benchmark_info_.has_value()) RETURN_IF_ERROR(benchmark_info_->TimeMarkDelta("executor_decode_and_sample"));
-    RETURN_IF_ERROR(executor_.Decode(output_tokens_));
-    if (benchmark_info_.has_value()) RETURN_IF_ERROR(benchmark_info_->TimeMarkDelta("executor_decode_and_sample"));
-    if (output_tokens_.NumElements() != 1) return InternalError("Unexpected number of decoded tokens.");
-    RETURN_IF_ERROR(detector_.ProcessTokens(output_tokens_.as<int32_t>(), 1));
-    return detector_.AllDone();
-  }
-  int token() const { return output_tokens_.as<int32_t>()[0]; }
-
- private:
-  LlmExecutor& executor_;
-  std::optional<BenchmarkInfo>& benchmark_info_;
-  StopTokenDetector detector_;
-  TensorBuffer output_tokens_;
+struct LoopLimits {
+  int forced_steps;    // benchmark's decode step count, 0 = none: then a stop sequence ends the loop
+  int max_num_tokens;  // KV-cache capacity in steps
 };
+
+LoopLimits LimitsOf(const LlmExecutor& executor, const std::optional<BenchmarkInfo>& benchmark_info) {
+  // An executor that cannot report its settings is taken to hold 4096 tokens (pipeline.cc:50-62).
+  auto settings = executor.GetExecutorSettings();
+  return LoopLimits{benchmark_info.has_value() ? benchmark_info->GetBenchmarkParams().num_decode_tokens : 0,
+                    settings.ok() ? settings->GetMaxNumTokens() : 4096};
+}
+
+LoopEnd Judge(const LoopLimits& limits, bool stop_tokens_seen, int steps_done, int current_step) {
+  if (limits.forced_steps == 0 && stop_tokens_seen) return LoopEnd::kStopTokens;
+  if (limits.forced_steps > 0 && steps_done >= limits.forced_steps) return LoopEnd::kStepBudget;
+  if (current_step >= limits.max_num_tokens) return LoopEnd::kCacheFull;
+  return LoopEnd::kGoOn;
+}
+
+// The loop both decode entry points share. Each step: Decode(tokens) with sampling inside the executor, timed as
+// the mark "executor_decode_and_sample" (pipeline.cc:160-227), the id shown to the stop detector (a private copy:
+// the caller's keeps its state) and to `emit`; `on_cache_full`, when given, hears of the cache limit before the
+// loop ends. A failed step is returned as it is, after `on_failure` (when given) has seen it.
+Status RunDecodeLoop(LlmExecutor& executor, StopTokenDetector detector, std::optional<BenchmarkInfo>& benchmark_info,
+                     const std::function<void(int)>& emit, const std::function<void(const Status&)>& on_failure,
+                     const std::function<void(const Status&)>& on_cache_full) {
+  static const char kMark[] = "executor_decode_and_sample";
+  const LoopLimits limits = LimitsOf(executor, benchmark_info);
+  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimeDecodeTurnStart());
+  TensorBuffer id_buffer = TensorBuffer::Create(ElementType::kInt32, {1, 1});
+  auto step = [&]() -> StatusOr<bool> {
+    if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimeMarkDelta(kMark));
+    RETURN_IF_ERROR(executor.Decode(id_buffer));
+    if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimeMarkDelta(kMark));
+    if (id_buffer.NumElements() != 1) return InternalError("Unexpected number of decoded tokens.");
+    RETURN_IF_ERROR(detector.ProcessTokens(id_buffer.as<int32_t>(), 1));
+    return detector.AllDone();
+  };
+  int steps_done = 0;
+  for (LoopEnd end = LoopEnd::kGoOn; end == LoopEnd::kGoOn;) {
+    const StatusOr<bool> stop_tokens_seen = step();
+    if (!stop_tokens_seen.ok()) {
+      if (on_failure) on_failure(stop_tokens_seen.status());
+      return stop_tokens_seen.status();
+    }
+    ++steps_done;
+    if (emit) emit(id_buffer.as<int32_t>()[0]);
+    ASSIGN_OR_RETURN(const int current_step, executor.GetCurrentStep());
+    end = Judge(limits, *stop_tokens_seen, steps_done, current_step);
+    if (end == LoopEnd::kCacheFull && on_cache_full) on_cache_full(InternalError("Maximum kv-cache size reached."));
+  }
+  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimeDecodeTurnEnd(steps_done));
+  return OkStatus();
+}
 
 }  // namespace
 
 StatusOr<int> Prefill(LlmExecutor& executor, std::vector<int> ids, int bos_token_id, bool wait_for_completion,
                       std::optional<BenchmarkInfo>& benchmark_info) {
-  int benchmark_prefill_token_count = 0;
-  if (benchmark_info.has_value()) {
-    benchmark_prefill_token_count = benchmark_info->GetBenchmarkParams().num_prefill_tokens;
-    RETURN_IF_ERROR(benchmark_info->TimePrefillTurnStart());
-  }
-  if (benchmark_prefill_token_count > 0) ids.resize(benchmark_prefill_token_count);
+  // A benchmark that names a prefill length decides the ids' count (cut, or padded with 0); otherwise the
+  // begin-of-sequence id goes in front (pipeline.cc:231-252).
+  const int forced = benchmark_info.has_value() ? benchmark_info->GetBenchmarkParams().num_prefill_tokens : 0;
+  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimePrefillTurnStart());
+  if (forced > 0) ids.resize(forced);
   else ids.insert(ids.begin(), bos_token_id);
-  const int max_num_tokens = TryGetMaxNumTokens(executor);
-  if (static_cast<int>(ids.size()) >= max_num_tokens)
-    return InvalidArgumentError("Input token ids are too long. Exceeding the maximum number of tokens allowed: " +
-                                std::to_string(ids.size()) + " >= " + std::to_string(max_num_tokens));
-  if (ids.empty()) return InternalError("Input token ids are empty.");
-  const int last_token_id = ids.back();
+
+  auto settings = executor.GetExecutorSettings();
+  const int max_num_tokens = settings.ok() ? settings->GetMaxNumTokens() : 4096;
   const int count = static_cast<int>(ids.size());
+  if (count >= max_num_tokens)
+    return InvalidArgumentError("Input token ids are too long. Exceeding the maximum number of tokens allowed: " +
+                                std::to_string(count) + " >= " + std::to_string(max_num_tokens));
+  if (count == 0) return InternalError("Input token ids are empty.");
+
   ExecutorPrefillParams params;
   params.SetWaitForCompletion(wait_for_completion);
-  RETURN_IF_ERROR(executor.Prefill(
-      ExecutorInputs(ExecutorTextData(TensorBuffer::CopyFrom(ElementType::kInt32, {1, count}, ids.data()))), params));
-  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimePrefillTurnEnd(ids.size()));
-  return last_token_id;
+  ExecutorInputs inputs(ExecutorTextData(TensorBuffer::CopyFrom(ElementType::kInt32, {1, count}, ids.data())));
+  RETURN_IF_ERROR(executor.Prefill(inputs, params));
+  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimePrefillTurnEnd(count));
+  return ids.back();
 }
 
 Status DecodeStreaming(LlmExecutor& executor, const StopTokenDetector& stop_token_detector,
                        std::optional<BenchmarkInfo>& benchmark_info, const std::function<void(int)>& on_next,
                        const std::function<void(const Status&)>& on_error) {
-  int benchmark_decode_token_count = 0;
-  if (benchmark_info.has_value()) {
-    benchmark_decode_token_count = benchmark_info->GetBenchmarkParams().num_decode_tokens;
-    RETURN_IF_ERROR(benchmark_info->TimeDecodeTurnStart());
-  }
-  int num_decoded_steps = 0;
-  const int max_num_tokens = TryGetMaxNumTokens(executor);
-  DecodeInternalSamplingOneStep run_one_step(executor, stop_token_detector, benchmark_info);
-  while (true) {
-    StatusOr<bool> hit_stop_tokens = run_one_step.Run();
-    if (!hit_stop_tokens.ok()) {
-      if (on_error) on_error(hit_stop_tokens.status());
-      return hit_stop_tokens.status();
-    }
-    ++num_decoded_steps;
-    if (on_next) on_next(run_one_step.token());
-    ASSIGN_OR_RETURN(const int current_step, executor.GetCurrentStep());
-    const auto stop = ShouldStop(*hit_stop_tokens, benchmark_decode_token_count, num_decoded_steps, current_step,
-                                 max_num_tokens);
-    if (stop.second && on_error) on_error(InternalError("Maximum kv-cache size reached."));
-    if (stop.first) break;
-  }
-  if (benchmark_info.has_value()) RETURN_IF_ERROR(benchmark_info->TimeDecodeTurnEnd(num_decoded_steps));
-  return OkStatus();
+  // The observer hears of failed steps and of the cache limit (pipeline.cc:320-367).
+  return RunDecodeLoop(executor, stop_token_detector, benchmark_info, on_next, on_error, on_error);
 }
 
 StatusOr<std::vector<int>> Decode(LlmExecutor& executor, const StopTokenDetector& stop_token_detector,
                                   std::optional<BenchmarkInfo>& benchmark_info) {
-  std::vector<int> tokens;
-  RETURN_IF_ERROR(DecodeStreaming(executor, stop_token_detector, benchmark_info,
-                                  [&](int id) { tokens.push_back(id); }, nullptr));
-  return tokens;
+  // No observer: the cache limit ends the loop silently (pipeline.cc:278-318).
+  std::vector<int> ids;
+  RETURN_IF_ERROR(RunDecodeLoop(executor, stop_token_detector, benchmark_info, [&ids](int id) { ids.push_back(id); },
+                                nullptr, nullptr));
+  return ids;
 }
 
 }  // namespace litert::lm
