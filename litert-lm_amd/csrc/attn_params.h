@@ -155,6 +155,9 @@ struct PrefillArgs {
   float* ws_acc;
   float* ws_ml;
   int32_t rows16;  // 1: the kernel on 16x16x32 MFMAs, two workgroups per compute unit; 0: the one on 32x32x16; < 0: by rule
+  // Work plan of the kernel on 16x16x32 MFMAs (device memory): [workgroups + 1] offsets into the item list, then
+  // two words per item, (unit, tile | part << 20), each workgroup's items in the order it runs them.
+  const int32_t* plan;
   uint16_t unit_order[128];
 };
 constexpr int kPrefillQueues = 2;                     // ticket queues; workgroup k draws from queue k % 2 first

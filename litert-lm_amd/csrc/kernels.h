@@ -32,10 +32,28 @@ struct PrefillSplit {
 };
 PrefillSplit plan_prefill_split(const PrefillArgs& args, int option);
 
+// Work plans of the prefill kernel on 16x16x32 MFMAs, kept by the handle: which workgroup runs which work items
+// in which order, computed on the host (longest processing time first over the workgroups: an item's time is
+// known from its number of key blocks) and cached by launch shape. A slot's device copy is rewritten only
+// after the last launch that reads it has finished (`used`); a slot whose launch was captured into a HIP graph
+// is kept for good (`pinned`: the graph may be replayed at any time).
+struct PrefillPlans {
+  static constexpr int kSlots = 4;
+  int32_t* d_words[kSlots] = {};
+  int32_t* h_words[kSlots] = {};  // pinned staging
+  size_t cap[kSlots] = {};        // words
+  hipEvent_t used[kSlots] = {};
+  int64_t key[kSlots][8] = {};
+  bool valid[kSlots] = {};
+  bool pinned[kSlots] = {};
+  int next = 0;
+};
+void free_prefill_plans(PrefillPlans* plans);
+
 // With args.kchunk > 0 the merge kernel follows the attention kernel (ev1 then marks the end of the
 // attention kernel alone).
-hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, hipStream_t stream,
-                          hipEvent_t ev0, hipEvent_t ev1);
+hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, PrefillPlans* plans,
+                          hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1);
 
 // Scatter n boundary-layout rows into the cache planes / gather them back.
 hipError_t launch_kv_append(const KvCopyArgs& args, hipStream_t stream);

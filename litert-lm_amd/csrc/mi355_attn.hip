@@ -83,6 +83,7 @@ struct mi355_attn {
   float* scales = nullptr;
   int32_t* d_window = nullptr;
   int32_t* d_sched = nullptr;  // prefill work-queue counters
+  PrefillPlans pf_plans;       // prefill work plans by launch shape
   float* d_pf_acc = nullptr;   // prefill key split: parts of split tiles, allocated on first use
   float* d_pf_ml = nullptr;
   size_t pf_rows = 0;          // rows (of head_dim / of 2 floats) the two hold
@@ -415,7 +416,7 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
       a.ws_acc = h->d_pf_acc;
       a.ws_ml = h->d_pf_ml;
     }
-    HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->stream, e0, e1));
+    HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, &h->pf_plans, h->stream, e0, e1));
   } else {
     // Row-wise path (fp32 and int8 caches): every query row is one decode item
     // whose key range ends at its own position.
@@ -605,6 +606,7 @@ void mi355_attn_destroy(mi355_attn* h) {
   if (h->scales) (void)hipFree(h->scales);
   if (h->d_window) (void)hipFree(h->d_window);
   if (h->d_sched) (void)hipFree(h->d_sched);
+  free_prefill_plans(&h->pf_plans);
   if (h->d_pf_acc) (void)hipFree(h->d_pf_acc);
   if (h->d_pf_ml) (void)hipFree(h->d_pf_ml);
   if (h->d_transform) (void)hipFree(h->d_transform);

@@ -620,11 +620,18 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
 // across the phases - is 3 to 10 % slower on the 26-layer launch: the exponentials
 // were already hidden by the other wave of the SIMD, and what the hand-placed order
 // adds in scheduling regions and waits costs more than the phases' ramps it removes.)
+// A read of read-only, wave-uniform data through the scalar cache (constant address space).
+__device__ __forceinline__ int32_t scalar_load(const int32_t* p) {
+  return *reinterpret_cast<const __attribute__((address_space(4))) int32_t*>(reinterpret_cast<uintptr_t>(p));
+}
+
 constexpr int kWaves16 = 4;
 constexpr int kRows16 = 16;
 constexpr int kSub16 = 2;       // sub-tiles of 16 query positions per wave
 constexpr int kKStages16 = 3, kVStages16 = 2;
-constexpr int kOpAhead = 4;     // LDS operand reads in flight ahead of their MFMAs
+// LDS operand reads in flight ahead of their MFMAs, scores and P.V (four each would not fit in 256 registers)
+constexpr int kOpAhead = 3;
+constexpr int kOpAheadV = 3;
 
 template <int D>
 constexpr int prefill16_lds_bytes() { return (kKStages16 + kVStages16) * 64 * D; }  // 80 KiB: two workgroups fill a CU's LDS
@@ -648,117 +655,140 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint8_t* const sm_k = smem;
   uint8_t* const sm_v = smem + kKStages16 * kBlockBytes;
-  // The ticket of the next item travels through the last K stage: every wave is done with the K
-  // ring once thread 0 is past the last barrier of an item, and no transfer writes that stage before
-  // the second barrier of the next item, when everybody has read the ticket.
-  volatile int* const sm_ticket = reinterpret_cast<volatile int*>(sm_k + kKStages16 * kBlockBytes - 16);
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
   const int hblocks = a.group / HPB;
   const int per_layer = a.geom.hkv * hblocks;
-  const int units = a.n_layers * per_layer;
-  const int tiles = (a.n + kStretch * PT - 1) / (kStretch * PT);
-  const int home = blockIdx.x & (kPrefillQueues - 1);
-  int tried = 0;
-  bool first_draw = true;
   const int smax = a.kchunk > 0 ? a.smax : 1;
   const float softcap = a.softcap;
   const float c = CAP ? 1.f : a.scale * kLog2e;
   const int pos_end = a.q_pos0 + a.n;
 
-  struct Item { int li, kvh, hb, tile, part, layer, window, wg_pos0, kb_lo, nblk_tile; };
-  auto item_of = [&](int qx, int ticket) {
+  // This workgroup's items, in the order the host planned them (no queue, no ticket: every wave reads the list).
+  const int32_t* const plan_items = a.plan + gridDim.x + 1;
+  const int item_end = scalar_load(a.plan + blockIdx.x + 1);
+
+  struct Item { int li, kvh, layer, window, wg_pos0, part, head, my_pos0, kb0, nblk; bool split; };
+  auto item_at = [&](int idx) {
     Item it;
-    const int qcnt = (units - qx + kPrefillQueues - 1) / kPrefillQueues;
-    const int per_tile = qcnt * smax;
-    const int ti = ticket / per_tile, r2 = ticket - ti * per_tile;
-    it.part = r2 / qcnt;
-    const int slot = qx + kPrefillQueues * (r2 - it.part * qcnt);
-    const int u = a.use_order ? a.unit_order[slot] : slot;
+    // (read through the scalar cache: a vector load here would make every item wait for all memory
+    // operations under way, the previous item's stores included)
+    const int u = scalar_load(plan_items + 2 * idx);
+    const int w1 = scalar_load(plan_items + 2 * idx + 1);
+    const int tile = w1 & 0xFFFFF;
+    it.part = w1 >> 20;
     it.li = u / per_layer;
     const int rem = u - it.li * per_layer;
     it.kvh = rem / hblocks;
-    it.hb = rem - it.kvh * hblocks;
-    it.tile = tiles - 1 - ti;
+    const int hb = rem - it.kvh * hblocks;
     it.layer = a.layer_begin + it.li;
-    it.window = a.layer_window[it.layer];
-    it.wg_pos0 = a.q_pos0 + it.tile * (kStretch * PT);
+    it.window = scalar_load(a.layer_window + it.layer);
+    it.wg_pos0 = a.q_pos0 + tile * (kStretch * PT);
     const int last_pos = min(it.wg_pos0 + kStretch * PT, pos_end) - 1;
-    it.kb_lo = 0;
-    if (it.window > 0 && it.wg_pos0 - it.window + 1 > 0) it.kb_lo = (it.wg_pos0 - it.window + 1) / kKeysPerBlock;
-    it.nblk_tile = last_pos / kKeysPerBlock - it.kb_lo + 1;
+    int kb_lo = 0;
+    if (it.window > 0 && it.wg_pos0 - it.window + 1 > 0) kb_lo = (it.wg_pos0 - it.window + 1) / kKeysPerBlock;
+    const int nblk_tile = last_pos / kKeysPerBlock - kb_lo + 1;
+    it.split = smax > 1 && nblk_tile > a.kchunk;
+    it.kb0 = kb_lo + (smax > 1 ? it.part * a.kchunk : 0);
+    it.nblk = smax > 1 ? min(a.kchunk, nblk_tile - it.part * a.kchunk) : nblk_tile;
+    it.head = it.kvh * a.group + hb * HPB + (wave % HPB);
+    it.my_pos0 = it.wg_pos0 + (wave / HPB) * kStretch;  // first of the wave's 32 positions
     return it;
   };
-
-  for (;;) {
-    if (tid == 0) {
-      int x = 0, t = -1;
-      while (tried < kPrefillQueues) {
-        x = (home + tried) & (kPrefillQueues - 1);
-        const int cnt = (units - x + kPrefillQueues - 1) / kPrefillQueues;
-        if (cnt > 0) {
-          const int home_wgs = ((int)gridDim.x - x + kPrefillQueues - 1) / kPrefillQueues;
-          if (first_draw && tried == 0) t = (int)blockIdx.x / kPrefillQueues;
-          else t = atomicAdd(a.sched + x, 1) + home_wgs;
-          first_draw = false;
-          if (t < cnt * tiles * smax) {
-            if (smax == 1) break;
-            const Item it = item_of(x, t);
-            if (it.part * a.kchunk < it.nblk_tile) break;
-            t = -1;
-            continue;
-          }
-          t = -1;
-        }
-        ++tried;
-      }
-      sm_ticket[0] = x;
-      sm_ticket[1] = t;
-    }
-    lds_barrier();  // also: every wave is done with the rings of the previous item
-    const int qx = __builtin_amdgcn_readfirstlane(sm_ticket[0]);
-    const int ticket = __builtin_amdgcn_readfirstlane(sm_ticket[1]);
-    if (ticket < 0) break;
-    const Item it = item_of(qx, ticket);
-    const int li = it.li, kvh = it.kvh, layer = it.layer, window = it.window;
-    const int head = kvh * a.group + it.hb * HPB + (wave % HPB);
-    const int my_pos0 = it.wg_pos0 + (wave / HPB) * kStretch;  // first of the wave's 32 positions
-    const uint8_t* kplane = a.cache + a.geom.plane_offset(layer, a.seq, kvh, 0);
-    const uint8_t* vplane = kplane + a.geom.plane_bytes;
-    const bool split_tile = smax > 1 && it.nblk_tile > a.kchunk;
-    const int kb_lo = it.kb_lo + (smax > 1 ? it.part * a.kchunk : 0);
-    const int nblk = smax > 1 ? min(a.kchunk, it.nblk_tile - it.part * a.kchunk) : it.nblk_tile;
-
-    auto fetch = [&](const uint8_t* plane, uint8_t* ring, int stages, int i) {
+  auto k_plane = [&](const Item& it) { return a.cache + a.geom.plane_offset(it.layer, a.seq, it.kvh, 0); };
+  // One 16 KiB block from a cache plane into a ring stage: every wave moves four 1 KiB pieces. The source is
+  // a wave-uniform address (scalar registers) plus the lane's 16-byte slot, so that the transfers need no
+  // vector arithmetic and no address registers of their own.
+  const uint32_t lane_slot = (uint32_t)lane * 16u;
+  auto fetch = [&](const uint8_t* plane, int block, uint8_t* stage) {
+    const uint8_t* const base = plane + (int64_t)block * kBlockBytes + wave * 1024;
 #pragma unroll
-      for (int t = 0; t < kXfers; ++t) {
-        const int off = (wave + kWaves16 * t) * 1024;
-        const uint8_t* src = plane + (int64_t)(kb_lo + i) * kBlockBytes + lane * 16 + off;
-        uint8_t* dst = ring + (i % stages) * kBlockBytes + off;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-      }
-    };
-    // Ring protocol, one barrier per block. Iteration i: K(i + 2) is asked for at
-    // the top (its stage held K(i - 1), read before the middle barrier of i - 1);
-    // scores and softmax of block i; every wave waits for its share of V(i) (asked
-    // for in the middle of i - 1; K(i + 1), older still, has then landed too);
-    // barrier; V(i + 1) is asked for (its stage held V(i - 1)); P.V of block i.
-    fetch(kplane, sm_k, kKStages16, 0);
-    fetch(vplane, sm_v, kVStages16, 0);
-    if (nblk > 1) fetch(kplane, sm_k, kKStages16, 1);
-
-    // Q^T operands: lane (n, g) holds, for sub-tile u and step j, channels 32 j + 8 g .. + 7 of query my_pos0 + 16 u + n
-    vec8 q[kSub16][NJ];
+    for (int t = 0; t < kXfers; ++t) {
+      const uint8_t* src = base + t * (kWaves16 * 1024) + lane_slot;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(stage + (wave + kWaves16 * t) * 1024),
+                                       16, 0, 0);
+    }
+  };
+  // Q^T operands: lane (n, g) holds, for sub-tile u and step j, channels 32 j + 8 g .. + 7 of query my_pos0 + 16 u + n.
+  // They are loaded behind the compiler's back (it would wait for ALL memory operations under way before the
+  // first use of a register loaded across the item loop): q_wait() below is the matching wait.
+  vec8 q[kSub16][NJ];
+  static_assert(NJ == 8, "load_q spells out eight steps");
+#define MI355_LOAD_Q(u, j) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "+v"(q[u][j]) : "v"(qrow), "n"(64 * (j)) : "memory")
+  auto load_q = [&](const Item& it) {
 #pragma unroll
     for (int u = 0; u < kSub16; ++u) {
-      const int row = min(my_pos0 + kRows16 * u + n - a.q_pos0, a.n - 1);  // rows past the end repeat the last one; never stored
-      const elem_t* qrow = reinterpret_cast<const elem_t*>(a.q) + (((int64_t)li * a.n + row) * a.hq + head) * D;
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) q[u][j] = *reinterpret_cast<const vec8*>(qrow + 32 * j + 8 * g);
+      const int row = min(it.my_pos0 + kRows16 * u + n - a.q_pos0, a.n - 1);  // rows past the end repeat the last one; never stored
+      const elem_t* qrow = reinterpret_cast<const elem_t*>(a.q) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + 8 * g;
+      MI355_LOAD_Q(u, 0); MI355_LOAD_Q(u, 1); MI355_LOAD_Q(u, 2); MI355_LOAD_Q(u, 3);
+      MI355_LOAD_Q(u, 4); MI355_LOAD_Q(u, 5); MI355_LOAD_Q(u, 6); MI355_LOAD_Q(u, 7);
     }
+  };
+#undef MI355_LOAD_Q
+  // After a wait that covers the query loads: from here on the compiler may read q.
+  auto q_ready = [&]() {
+#pragma unroll
+    for (int u = 0; u < kSub16; ++u)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) asm volatile("" : "+v"(q[u][j]));
+  };
+
+  // The key blocks of all items of this workgroup form one stream through the rings: block s of the stream
+  // sits in K stage s % 3 and V stage s % 2, whatever item it belongs to. While block s is worked on, K(s + 2)
+  // is asked for after the scores (its stage held K(s - 1), last read before the barrier of block s - 1) and
+  // V(s + 1) after the barrier of block s (its stage held V(s - 1), last read before that barrier) - also
+  // when those blocks belong to the next item, whose first blocks, and whose queries (loaded into the
+  // registers the last scores have just freed), are therefore under way while this item's last P.V and
+  // its store run. Nothing waits and no barrier stands between two items.
+  int idx = scalar_load(a.plan + blockIdx.x);
+  if (idx >= item_end) return;
+  Item it = item_at(idx);
+  int ks = 0;        // K stage of the block being worked on
+  int kfs = 0;       // K stage the next block asked for goes to
+  int vs = 0;        // V stage of the block being worked on
+  int kreq = 0;      // K blocks of the current item already asked for when it starts (0 .. 2)
+  bool v_asked = false, q_loaded = false, k0_landed = false;
+  int stores_after_q = 0;  // store instructions certainly issued after the latest query loads (never more than were)
+
+  for (;;) {
+    const bool has_next = idx + 1 < item_end;
+    const Item nx = item_at(has_next ? idx + 1 : idx);
+    const int nblk = it.nblk;
+    const int lim = nblk + (has_next ? min(2, nx.nblk) : 0);  // stream blocks (counted from this item's first) that may be asked for
+    const uint8_t* const kplane = k_plane(it);
+    const uint8_t* const vplane = kplane + a.geom.plane_bytes;
+    const uint8_t* const kplane_nx = k_plane(nx);
+    auto ask_k = [&](int r) {  // r: stream block counted from this item's first
+      if (r < nblk) fetch(kplane, it.kb0 + r, sm_k + kfs * kBlockBytes);
+      else fetch(kplane_nx, nx.kb0 + (r - nblk), sm_k + kfs * kBlockBytes);
+      kfs = kfs == kKStages16 - 1 ? 0 : kfs + 1;
+    };
+    // What the previous item has not asked for already (everything, for a workgroup's first item).
+    int req = kreq;
+    if (req < 1) { ask_k(0); req = 1; }
+    if (!v_asked) fetch(vplane, it.kb0, sm_v + vs * kBlockBytes);
+    if (req < 2 && nblk > 1) { ask_k(1); req = 2; }
+    if (!q_loaded) load_q(it);
+    if (!k0_landed) {
+      // K(0) has to be there for everybody: a workgroup's first item, or one after a one-block item, whose K(0)
+      // was asked for only during that item's single block. (Everything is waited for, the queries too: on the
+      // other path into the scores they were loaded long ago, and the wait the compiler puts there is sized
+      // for that path.)
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      lds_barrier();
+    } else {
+      // The queries were loaded during the previous item's last P.V; since then: V(0) of this item (one
+      // block's transfers) and that item's stores. Memory operations complete in the order issued.
+      if (stores_after_q >= 2 * NL) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers + 2 * NL));
+      else if (stores_after_q >= NL) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers + NL));
+      else if (stores_after_q >= NL / 2) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers + NL / 2));
+      else __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
+    }
+    q_ready();
+
     f4 acc[kSub16][NL];
 #pragma unroll
     for (int u = 0; u < kSub16; ++u)
@@ -767,18 +797,13 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
     float m_run[kSub16], l_run[kSub16];
 #pragma unroll
     for (int u = 0; u < kSub16; ++u) { m_run[u] = -INFINITY; l_run[u] = 0.f; }
+    const int window = it.window, my_pos0 = it.my_pos0;
     const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
     const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
-    // K(0) has to be there for everybody (the query loads, issued last, may still be under way;
-    // the compiler waits for those where it needs them)
-    __builtin_amdgcn_s_waitcnt(wait_vm(kSub16 * NJ));
-    lds_barrier();
 
     for (int i = 0; i < nblk; ++i) {
-      const bool more_k = i + 2 < nblk, more_v = i + 1 < nblk;
-      if (more_k) fetch(kplane, sm_k, kKStages16, i + 2);
-      const uint8_t* kb = sm_k + (i % kKStages16) * kBlockBytes + lane * 16;
-      const uint8_t* vb = sm_v + (i % kVStages16) * kBlockBytes + lane * 16;
+      const uint8_t* kb = sm_k + ks * kBlockBytes + lane * 16;
+      const uint8_t* vb = sm_v + vs * kBlockBytes + lane * 16;
       f4 sc[kSub16][2];
 #pragma unroll
       for (int u = 0; u < kSub16; ++u)
@@ -798,9 +823,21 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
           for (int u = 0; u < kSub16; ++u) sc[u][T] = mfma(kop[st % kOpAhead], q[u][j], sc[u][T]);
           if (st + kOpAhead < 2 * NJ) kop[st % kOpAhead] = k_at(st + kOpAhead);
         }
+        // keep that order: kOpAhead reads, then two MFMAs and one read per step (left alone, the scheduler
+        // saves registers by reading every operand right before its use, and each step waits for LDS)
+        __builtin_amdgcn_sched_group_barrier(0x100, kOpAhead, 0);
+#pragma unroll
+        for (int st = 0; st < 2 * NJ; ++st) {
+          __builtin_amdgcn_sched_group_barrier(0x008, kSub16, 0);
+          if (st + kOpAhead < 2 * NJ) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
       }
+      // K two blocks ahead in the stream (normally one block; two after a one-block item's only scores)
+      int asked = 0;
+      if (req <= i + 2 && req < lim) { ask_k(req); ++req; ++asked; }
+      if (req <= i + 2 && req < lim) { ask_k(req); ++req; ++asked; }
       // score sc[u][T][e]: key key0 + 16 T + 4 g + e against query my_pos0 + 16 u + n
-      const int key0 = (kb_lo + i) * kKeysPerBlock;
+      const int key0 = (it.kb0 + i) * kKeysPerBlock;
       const bool all_vis = key0 + kKeysPerBlock - 1 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim;
       h8 p_hi[kSub16];
 #pragma unroll
@@ -845,78 +882,98 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
           for (int db = 0; db < NL; ++db) acc[u][db] *= alpha;
         }
       }
-      // this wave's share of V(i) (and of K(i + 1)) has landed; K(i + 2) may be under way
-      if (more_k) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
-      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      // This wave's share of V(i) and of K(i + 1) has landed; what was asked for after these scores may be under way.
+      if (asked == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+      else if (asked == 1) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
+      else __builtin_amdgcn_s_waitcnt(wait_vm(2 * kXfers));
       lds_barrier();
-      if (more_v) fetch(vplane, sm_v, kVStages16, i + 1);
+      const bool last = i + 1 == nblk;
+      if (!last) fetch(vplane, it.kb0 + i + 1, sm_v + (vs ^ 1) * kBlockBytes);
+      else if (has_next) {
+        load_q(nx);  // the scores of this item are done with the query registers
+        fetch(kplane_nx + a.geom.plane_bytes, nx.kb0, sm_v + (vs ^ 1) * kBlockBytes);
+      }
       {
-        h8 vop[kOpAhead];
+        h8 vop[kOpAheadV];
 #pragma unroll
-        for (int st = 0; st < kOpAhead; ++st) vop[st] = *reinterpret_cast<const h8*>(vb + st * 1024);
+        for (int st = 0; st < kOpAheadV; ++st) vop[st] = *reinterpret_cast<const h8*>(vb + st * 1024);
 #pragma unroll
         for (int db = 0; db < NL; ++db) {
 #pragma unroll
           for (int u = 0; u < kSub16; ++u) {
-            acc[u][db] = mfma16_f16(vop[db % kOpAhead], p_hi[u], acc[u][db]);
+            acc[u][db] = mfma16_f16(vop[db % kOpAheadV], p_hi[u], acc[u][db]);
           }
-          if (db + kOpAhead < NL) vop[db % kOpAhead] = *reinterpret_cast<const h8*>(vb + (db + kOpAhead) * 1024);
+          if (db + kOpAheadV < NL) vop[db % kOpAheadV] = *reinterpret_cast<const h8*>(vb + (db + kOpAheadV) * 1024);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, kOpAheadV, 0);
+#pragma unroll
+        for (int db = 0; db < NL; ++db) {
+          __builtin_amdgcn_sched_group_barrier(0x008, kSub16, 0);
+          if (db + kOpAheadV < NL) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
       }
-      // (no barrier here: the next one, in the middle of iteration i + 1, is passed only when every
+      ks = ks == kKStages16 - 1 ? 0 : ks + 1;
+      vs ^= 1;
+      // (no barrier here: the next one, in the middle of the stream's next block, is passed only when every
       // wave is done with this P.V, and V(i)'s stage is written no earlier than that)
     }
 
-    // ---- store: lane (n, g) holds channels 16 db + 4 g .. + 3 of query my_pos0 + 16 u + n
+    // ---- store, straight from the registers (the rings belong to the stream): lane (n, g) holds channels
+    // 16 db + 4 g .. + 3 of query my_pos0 + 16 u + n
+    stores_after_q = 0;
 #pragma unroll
     for (int u = 0; u < kSub16; ++u) {
       float l_tot = wave_xor_add(l_run[u], 16);
       l_tot = wave_xor_add(l_tot, 32);
       const int row = my_pos0 + kRows16 * u + n - a.q_pos0;
+      // (lane n = 0 has a row to store: the wave issues the sub-tile's store instructions, NL / 2 of 16 bytes, or
+      // NL + 1 for a part of a split tile)
+      if (wave_pos0 + kRows16 * u - a.q_pos0 < a.n) stores_after_q += it.split ? NL : NL / 2;
       if (row < a.n) {
-        if (split_tile) {
-          const int64_t slot = (((int64_t)li * a.n + row) * a.hq + head) * smax + it.part;
+        if (it.split) {
+          const int64_t slot = (((int64_t)it.li * a.n + row) * a.hq + it.head) * smax + it.part;
           float* prow = a.ws_acc + slot * D + 4 * g;
 #pragma unroll
           for (int db = 0; db < NL; ++db) *reinterpret_cast<f4*>(prow + 16 * db) = acc[u][db];
           if (g == 0) *reinterpret_cast<float2*>(a.ws_ml + slot * 2) = float2{m_run[u], l_tot};
         }
       }
-      if (!split_tile) {
-        // Whole rows through LDS (the K ring is idle: every wave has passed the last barrier of the
-        // loop; each wave has a patch of its own, 16 rows padded to 528 bytes, below the ticket), then
-        // two 512-byte rows per store instruction.
-        constexpr int kRowStride = 2 * D + 16;
-        static_assert(kWaves16 * kRows16 * kRowStride <= kKStages16 * kBlockBytes - 16, "patches below the ticket");
-        uint8_t* const patch = sm_k + wave * (kRows16 * kRowStride);
+      if (!it.split) {
+        // Pairs of channel tiles trade halves between the lanes g and g ^ 1 of a query (v_permlane16_swap), so
+        // that a lane ends up with 8 consecutive channels, 16 bytes, and the four lanes of a query with 64
+        // consecutive bytes per store instruction (8-byte pieces straight from the MFMA layout cost four
+        // times the write requests). Every lane takes part in the trade; only rows that exist are stored.
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        uint32_t packed[NL][2];
 #pragma unroll
         for (int db = 0; db < NL; ++db) {
           elem_t o[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = (elem_t)(acc[u][db][e] * inv);
-          *reinterpret_cast<u2*>(patch + n * kRowStride + (16 * db + 4 * g) * 2) = *reinterpret_cast<const u2*>(o);
+          const u2 w = *reinterpret_cast<const u2*>(o);
+          packed[db][0] = w[0];
+          packed[db][1] = w[1];
         }
-        // (the patch is private to the wave and LDS operations of a wave stay in order: no barrier)
-        const int row_base = my_pos0 + kRows16 * u - a.q_pos0;
-        const int chunk = lane & 31, hh = lane >> 5;
+        // lanes g = 0, 2 keep tile 2k (channels 32k + 4g .. + 7), lanes g = 1, 3 tile 2k + 1 (32k + 16 + 4(g - 1) .. + 7)
+        const int first = (g & 1) * 16 + (g >> 1) * 8;
+        elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + first;
 #pragma unroll
-        for (int jj = 0; jj < kRows16 / 2; ++jj) {
-          const int r = 2 * jj + hh;
-          const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStride + chunk * 16);
-          if (row_base + r < a.n) {
-            elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row_base + r) * a.hq + head) * D;
-            *reinterpret_cast<u4*>(orow + chunk * 8) = w;
-          }
+        for (int k = 0; k < NL / 2; ++k) {
+          const auto lo = __builtin_amdgcn_permlane16_swap(packed[2 * k][0], packed[2 * k + 1][0], false, false);
+          const auto hi = __builtin_amdgcn_permlane16_swap(packed[2 * k][1], packed[2 * k + 1][1], false, false);
+          const u4 w = {lo[0], hi[0], lo[1], hi[1]};
+          if (row < a.n) *reinterpret_cast<u4*>(orow + 32 * k) = w;
         }
       }
     }
-  }  // next work item
 
-  if (tid == 0) {
-    const int done = atomicAdd(a.sched + kPrefillQueues, 1);
-    if (done == (int)gridDim.x - 1)
-      for (int i = 0; i < kPrefillSchedInts; ++i) atomicExch(a.sched + i, 0);
+    if (!has_next) break;
+    kreq = req - nblk;
+    v_asked = true;
+    q_loaded = true;
+    k0_landed = nblk >= 2;  // then K(0) of the next item was asked for a block before this item's last barrier
+    it = nx;
+    ++idx;
   }
 }
 
@@ -990,8 +1047,129 @@ hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEv
                          : launch_variant<DT, D, HPB, false>(a, grid, stream, ev0, ev1);
 }
 
+// Key blocks of tile `t` of a layer with window `w` (0: global): the kernels' own arithmetic.
+int tile_key_blocks(const PrefillArgs& a, int rows_per_tile, int w, int t) {
+  const int p0 = a.q_pos0 + t * rows_per_tile;
+  const int last = std::min(p0 + rows_per_tile, a.q_pos0 + a.n) - 1;
+  const int lo = (w > 0 && p0 - w + 1 > 0) ? (p0 - w + 1) / kKeysPerBlock : 0;
+  return last / kKeysPerBlock - lo + 1;
+}
+
+// The work plan of a launch on `wgs` workgroups: items are dealt out longest first, each to the workgroup that
+// would be done with it earliest. The clock is a model of the measured launch (MI355X, 26 layers x 1024 tokens):
+// with two workgroups per compute unit (wgs == 2 * cus) the one the dispatcher places first (index < cus) has
+// its first loads served first and is at its first key block after about 5.7 us, the second after about 9.8 us;
+// sharing the compute unit, the first gets through a key block in about 2.1 us, the second in 2.45 us; an item
+// costs about 3 us besides its blocks (start, store). Both workgroups of a compute unit should finish together:
+// a workgroup left alone runs faster (1.5 us per block) but the compute unit as a whole slower than the pair.
+// With one workgroup per compute unit or fewer, all workgroups are alike.
+constexpr long kPlanMaxItems = 1L << 22;
+void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::vector<int32_t>* words) {
+  const int rows_per_tile = kStretch * (4 / hpb);
+  const int tiles = (a.n + rows_per_tile - 1) / rows_per_tile;
+  const int per_layer = a.geom.hkv * (a.group / hpb);
+  struct It { int32_t unit, w1, blocks; };
+  std::vector<It> items;
+  for (int li = 0; li < a.n_layers; ++li) {
+    const int w = a.host_window[a.layer_begin + li];
+    for (int t = 0; t < tiles; ++t) {
+      const int nblk = tile_key_blocks(a, rows_per_tile, w, t);
+      const int parts = a.kchunk > 0 ? (nblk + a.kchunk - 1) / a.kchunk : 1;
+      for (int part = 0; part < parts; ++part) {
+        const int blocks = a.kchunk > 0 ? std::min(a.kchunk, nblk - part * a.kchunk) : nblk;
+        for (int r = 0; r < per_layer; ++r) items.push_back(It{li * per_layer + r, t | (part << 20), blocks});
+      }
+    }
+  }
+  std::stable_sort(items.begin(), items.end(), [](const It& x, const It& y) { return x.blocks > y.blocks; });
+  // times in units of 0.05 us
+  constexpr long kFirstStart = 114, kSecondStart = 196, kFirstBlock = 42, kSecondBlock = 49, kItem = 60;
+  const bool paired = cus > 0 && wgs > cus;
+  // (time done, workgroup) min-heaps: the first-placed workgroups and the second-placed ones
+  using Entry = std::pair<long, int>;
+  auto later = [](const Entry& x, const Entry& y) { return x > y; };
+  std::vector<Entry> first, second;
+  for (int g = 0; g < wgs; ++g) {
+    if (paired && g >= cus) second.push_back({kSecondStart, g});
+    else first.push_back({paired ? kFirstStart : 0L, g});
+  }
+  std::make_heap(first.begin(), first.end(), later);
+  std::make_heap(second.begin(), second.end(), later);
+  std::vector<int> owner(items.size());
+  std::vector<int> count(wgs, 0);
+  for (size_t i = 0; i < items.size(); ++i) {
+    const long t1 = first.front().first + items[i].blocks * kFirstBlock + kItem;
+    const long t2 = second.empty() ? -1 : second.front().first + items[i].blocks * kSecondBlock + kItem;
+    std::vector<Entry>& heap = (t2 >= 0 && t2 < t1) ? second : first;
+    std::pop_heap(heap.begin(), heap.end(), later);
+    heap.back().first = &heap == &first ? t1 : t2;
+    owner[i] = heap.back().second;
+    ++count[owner[i]];
+    std::push_heap(heap.begin(), heap.end(), later);
+  }
+  words->assign((size_t)wgs + 1 + 2 * items.size(), 0);
+  int32_t* offs = words->data();
+  for (int g = 0; g < wgs; ++g) offs[g + 1] = offs[g] + count[g];
+  std::vector<int> fill(offs, offs + wgs);
+  int32_t* list = words->data() + wgs + 1;
+  for (size_t i = 0; i < items.size(); ++i) {
+    const int at = fill[owner[i]]++;
+    list[2 * at] = items[i].unit;
+    list[2 * at + 1] = items[i].w1;
+  }
+}
+
+void release_plan_slot(PrefillPlans* p, int s) {
+  if (p->d_words[s]) (void)hipFree(p->d_words[s]);
+  if (p->h_words[s]) (void)hipHostFree(p->h_words[s]);
+  p->d_words[s] = p->h_words[s] = nullptr;
+  p->cap[s] = 0;
+  p->valid[s] = false;
+}
+
+// Device copy of the plan for this launch shape: a cached one, or a new one built into the next slot and copied
+// on `stream` ahead of the launch.
+hipError_t plan_for(const PrefillArgs& a, int hpb, int wgs, int cus, PrefillPlans* p, hipStream_t stream, int* slot_out) {
+  const int64_t key[8] = {a.layer_begin, a.n_layers, a.q_pos0, a.n, a.kchunk, wgs, hpb, a.seq};
+  for (int s = 0; s < PrefillPlans::kSlots; ++s)
+    if (p->valid[s] && std::equal(key, key + 8, p->key[s])) {
+      *slot_out = s;
+      return hipSuccess;
+    }
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  hipError_t e = hipStreamIsCapturing(stream, &capturing);
+  if (e != hipSuccess) return e;
+  if (capturing != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;  // run the shape once before capturing it
+  int s = -1;
+  for (int k = 0; k < PrefillPlans::kSlots && s < 0; ++k) {
+    const int cand = (p->next + k) % PrefillPlans::kSlots;
+    if (!p->pinned[cand]) s = cand;
+  }
+  if (s < 0) return hipErrorOutOfMemory;  // every slot belongs to a captured graph
+  p->next = (s + 1) % PrefillPlans::kSlots;
+  if (!p->used[s] && (e = hipEventCreateWithFlags(&p->used[s], hipEventDisableTiming)) != hipSuccess) return e;
+  if ((e = hipEventSynchronize(p->used[s])) != hipSuccess) return e;  // the last launch that read this slot is over
+  p->valid[s] = false;
+  std::vector<int32_t> words;
+  build_prefill_plan(a, hpb, wgs, cus, &words);
+  if (p->cap[s] < words.size()) {
+    release_plan_slot(p, s);
+    const size_t cap = words.size() + words.size() / 2;
+    if ((e = hipMalloc(&p->d_words[s], cap * sizeof(int32_t))) != hipSuccess) return e;
+    if ((e = hipHostMalloc(&p->h_words[s], cap * sizeof(int32_t))) != hipSuccess) return e;
+    p->cap[s] = cap;
+  }
+  std::copy(words.begin(), words.end(), p->h_words[s]);
+  e = hipMemcpyAsync(p->d_words[s], p->h_words[s], words.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream);
+  if (e != hipSuccess) return e;
+  std::copy(key, key + 8, p->key[s]);
+  p->valid[s] = true;
+  *slot_out = s;
+  return hipSuccess;
+}
+
 template <int DT, int D>
-hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int G = a.group;
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
   const int pt = 4 / hpb;
@@ -1052,13 +1230,28 @@ hipError_t launch_typed(const PrefillArgs& a, hipStream_t stream, hipEvent_t ev0
   // per CU) when there are at least two work items per CU, else the one on 32x32x16 MFMAs, whose
   // single workgroup per CU gets through an item in half the time.
   b.rows16 = a.rows16 < 0 ? (all_items >= 2L * cus ? 1 : 0) : a.rows16;
+  // (the planned kernel needs the host's copy of the windows, and a plan of bounded size)
+  if (b.rows16 == 1 && (!a.host_window || all_items > kPlanMaxItems)) b.rows16 = 0;
   const int slots = b.rows16 == 1 ? 2 * cus : cus;
   int wgs = all_items < slots ? (int)all_items : slots;
   if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
   const dim3 grid(wgs, 1, 1);
+  int plan_slot = -1;
+  if (b.rows16 == 1) {
+    hipError_t pe = plan_for(a, hpb, wgs, cus, plans, stream, &plan_slot);
+    if (pe != hipSuccess) return pe;
+    b.plan = plans->d_words[plan_slot];
+  }
   hipError_t err = hpb == 4   ? launch_hpb<DT, D, 4>(b, grid, stream, ev0, ev1)
                    : hpb == 2 ? launch_hpb<DT, D, 2>(b, grid, stream, ev0, ev1)
                               : launch_hpb<DT, D, 1>(b, grid, stream, ev0, ev1);
+  if (err == hipSuccess && plan_slot >= 0) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    err = hipStreamIsCapturing(stream, &capturing);
+    // (a captured launch keeps its plan for as long as the graph may be replayed: the slot is never reused)
+    if (err == hipSuccess && capturing == hipStreamCaptureStatusNone) err = hipEventRecord(plans->used[plan_slot], stream);
+    else if (err == hipSuccess) plans->pinned[plan_slot] = true;
+  }
   if (err != hipSuccess || a.kchunk <= 0) return err;
   hipLaunchKernelGGL((prefill_merge_kernel<DT, D>), dim3(a.hq, a.n, a.n_layers), dim3(D), 0, stream, b, kStretch * pt);
   return hipGetLastError();
@@ -1110,12 +1303,23 @@ bool prefill_supported(int kv_dtype, int io_dtype, int head_dim) {
   return head_dim == 256 && kv_dtype == io_dtype && (kv_dtype == kF16 || kv_dtype == kBF16);
 }
 
-hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, hipStream_t stream, hipEvent_t ev0,
-                          hipEvent_t ev1) {
+hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, PrefillPlans* plans, hipStream_t stream,
+                          hipEvent_t ev0, hipEvent_t ev1) {
   (void)io_dtype;
-  if (kv_dtype == kF16) return launch_typed<kF16, 256>(a, stream, ev0, ev1);
-  if (kv_dtype == kBF16) return launch_typed<kBF16, 256>(a, stream, ev0, ev1);
+  if (kv_dtype == kF16) return launch_typed<kF16, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kBF16) return launch_typed<kBF16, 256>(a, plans, stream, ev0, ev1);
   return hipErrorInvalidValue;
+}
+
+void free_prefill_plans(PrefillPlans* p) {
+  for (int s = 0; s < PrefillPlans::kSlots; ++s) {
+    if (p->d_words[s]) (void)hipFree(p->d_words[s]);
+    if (p->h_words[s]) (void)hipHostFree(p->h_words[s]);
+    if (p->used[s]) (void)hipEventDestroy(p->used[s]);
+    p->d_words[s] = p->h_words[s] = nullptr;
+    p->used[s] = nullptr;
+    p->valid[s] = false;
+  }
 }
 
 }  // namespace mi355
