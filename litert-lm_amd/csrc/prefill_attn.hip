@@ -766,18 +766,22 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       else fetch(kplane_nx, nx.kb0 + (r - nblk), sm_k + kfs * kBlockBytes);
       kfs = kfs == kKStages16 - 1 ? 0 : kfs + 1;
     };
-    // What the previous item has not asked for already (everything, for a workgroup's first item).
+    // What the previous item has not asked for already: everything, for a workgroup's first item, whose queries
+    // and first K block go first, so that its first scores need not wait for V(0) and K(1) as well (at the start
+    // of a launch every workgroup asks at once and the loads are served at the rate of the memory).
+    const bool first_item = !q_loaded;
+    if (first_item) load_q(it);
     int req = kreq;
     if (req < 1) { ask_k(0); req = 1; }
-    if (!v_asked) fetch(vplane, it.kb0, sm_v + vs * kBlockBytes);
-    if (req < 2 && nblk > 1) { ask_k(1); req = 2; }
-    if (!q_loaded) load_q(it);
+    int after_k0 = 0;  // blocks asked for after K(0)
+    if (!v_asked) { fetch(vplane, it.kb0, sm_v + vs * kBlockBytes); ++after_k0; }
+    if (req < 2 && nblk > 1) { ask_k(1); req = 2; ++after_k0; }
     if (!k0_landed) {
       // K(0) has to be there for everybody: a workgroup's first item, or one after a one-block item, whose K(0)
-      // was asked for only during that item's single block. (Everything is waited for, the queries too: on the
-      // other path into the scores they were loaded long ago, and the wait the compiler puts there is sized
-      // for that path.)
-      __builtin_amdgcn_s_waitcnt(0x0F70);
+      // was asked for only during that item's single block (then everything is waited for: rare).
+      if (first_item && after_k0 == 2) __builtin_amdgcn_s_waitcnt(wait_vm(2 * kXfers));
+      else if (first_item && after_k0 == 1) __builtin_amdgcn_s_waitcnt(wait_vm(kXfers));
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
       lds_barrier();
     } else {
       // The queries were loaded during the previous item's last P.V; since then: V(0) of this item (one
