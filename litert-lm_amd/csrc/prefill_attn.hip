@@ -1089,24 +1089,69 @@ void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::ve
   // times in units of 0.05 us
   constexpr long kFirstStart = 114, kSecondStart = 196, kFirstBlock = 42, kSecondBlock = 49, kItem = 60;
   const bool paired = cus > 0 && wgs > cus;
-  // (time done, workgroup) min-heaps: the first-placed workgroups and the second-placed ones
+  // Workgroup g runs on XCD g % kXcds (the dispatcher deals workgroups out round robin), each XCD with an L2 of
+  // its own: a layer's items go to the workgroups of one XCD, so that its K / V planes are pulled into one L2
+  // instead of all eight - unless that XCD is behind the best workgroup anywhere by more than kStray, then the
+  // item strays (layers differ in work, and 26 layers do not divide by 8). Layers are dealt to the XCDs heaviest
+  // first, each to the XCD with the least work so far.
+  constexpr int kXcds = 8;
+  constexpr long kStray = 60;
+  const int xcds = wgs >= 4 * kXcds ? kXcds : 1;
+  std::vector<int> home(a.n_layers, 0);
+  if (xcds > 1) {
+    std::vector<long> layer_work(a.n_layers, 0), xcd_work(xcds, 0);
+    for (const It& it : items) layer_work[it.unit / per_layer] += it.blocks;
+    std::vector<int> by_work(a.n_layers);
+    for (int li = 0; li < a.n_layers; ++li) by_work[li] = li;
+    std::stable_sort(by_work.begin(), by_work.end(), [&](int x, int y) { return layer_work[x] > layer_work[y]; });
+    for (int li : by_work) {
+      const int x = (int)(std::min_element(xcd_work.begin(), xcd_work.end()) - xcd_work.begin());
+      home[li] = x;
+      xcd_work[x] += layer_work[li];
+    }
+  }
+  // (time done, workgroup) min-heaps per XCD: the first-placed workgroups and the second-placed ones
   using Entry = std::pair<long, int>;
   auto later = [](const Entry& x, const Entry& y) { return x > y; };
-  std::vector<Entry> first, second;
+  std::vector<std::vector<Entry>> first(xcds), second(xcds);
   for (int g = 0; g < wgs; ++g) {
-    if (paired && g >= cus) second.push_back({kSecondStart, g});
-    else first.push_back({paired ? kFirstStart : 0L, g});
+    if (paired && g >= cus) second[g % xcds].push_back({kSecondStart, g});
+    else first[g % xcds].push_back({paired ? kFirstStart : 0L, g});
   }
-  std::make_heap(first.begin(), first.end(), later);
-  std::make_heap(second.begin(), second.end(), later);
+  for (int x = 0; x < xcds; ++x) {
+    std::make_heap(first[x].begin(), first[x].end(), later);
+    std::make_heap(second[x].begin(), second[x].end(), later);
+  }
   std::vector<int> owner(items.size());
   std::vector<int> count(wgs, 0);
   for (size_t i = 0; i < items.size(); ++i) {
-    const long t1 = first.front().first + items[i].blocks * kFirstBlock + kItem;
-    const long t2 = second.empty() ? -1 : second.front().first + items[i].blocks * kSecondBlock + kItem;
-    std::vector<Entry>& heap = (t2 >= 0 && t2 < t1) ? second : first;
+    // the best workgroup of an XCD for this item: (time it would be done, which heap)
+    auto best_of = [&](int x) {
+      long t = -1;
+      std::vector<Entry>* heap = nullptr;
+      if (!first[x].empty()) {
+        t = first[x].front().first + items[i].blocks * kFirstBlock + kItem;
+        heap = &first[x];
+      }
+      if (!second[x].empty()) {
+        const long t2 = second[x].front().first + items[i].blocks * kSecondBlock + kItem;
+        if (t < 0 || t2 < t) {
+          t = t2;
+          heap = &second[x];
+        }
+      }
+      return std::make_pair(t, heap);
+    };
+    auto pick = best_of(home[items[i].unit / per_layer]);
+    auto best = pick;
+    for (int x = 0; x < xcds; ++x) {
+      const auto other = best_of(x);
+      if (other.second && (!best.second || other.first < best.first)) best = other;
+    }
+    if (!pick.second || best.first + kStray < pick.first) pick = best;
+    std::vector<Entry>& heap = *pick.second;
     std::pop_heap(heap.begin(), heap.end(), later);
-    heap.back().first = &heap == &first ? t1 : t2;
+    heap.back().first = pick.first;
     owner[i] = heap.back().second;
     ++count[owner[i]];
     std::push_heap(heap.begin(), heap.end(), later);
