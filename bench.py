@@ -389,7 +389,7 @@ def pipeline_report(X, device_resident):
     import re
     layers = 26
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
-    kw = {"device_resident": True} if device_resident else {}
+    kw = {"device_resident": bool(device_resident)}
     with X.HipLlmExecutor(layers, 4, 1, 64, 2048, runner_lengths=(1024,), layer_window=windows, fp16=True,
                           pre_attention=True, **kw) as ex:
         r = X.run_benchmark(ex, [3, 1, 4, 1, 5, 9, 2, 6], 1024, 256)
