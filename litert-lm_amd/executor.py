@@ -315,6 +315,28 @@ SECTION_NONE, SECTION_BINARY, SECTION_DEPRECATED, SECTION_TFLITE, SECTION_SP_TOK
     SECTION_HF_TOKENIZER_ZLIB = range(7)
 
 
+def model_file(path, preset_max_num_tokens=0) -> dict:
+    """What an executor takes from a .litertlm file: the section map by kind and the token capacity (the settings'
+    own value if `preset_max_num_tokens` is set, else the file's LlmMetadata.max_num_tokens, else 4096)."""
+    import json
+    lib().hle_model_file.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p)]
+    text, err = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = lib().hle_model_file(str(path).encode(), preset_max_num_tokens, ctypes.byref(text), ctypes.byref(err))
+    out = _take_text(text.value)
+    _check(rc, err)
+    return json.loads(out)
+
+
+def proto_int32_field(message: bytes, field_number: int) -> int:
+    lib().hle_proto_int32_field.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32),
+                                            ctypes.POINTER(ctypes.c_void_p)]
+    buf = ctypes.create_string_buffer(bytes(message), len(message))
+    value, err = ctypes.c_int32(), ctypes.c_void_p()
+    _check(lib().hle_proto_int32_field(ctypes.cast(buf, ctypes.c_void_p), len(message), field_number, ctypes.byref(value),
+                                       ctypes.byref(err)), err)
+    return value.value
+
+
 def litertlm_header(path=None, data=None) -> dict:
     """Header of a .litertlm file (or of a bytes object): version, system metadata, section map."""
     import json

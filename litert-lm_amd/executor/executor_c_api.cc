@@ -13,6 +13,7 @@
 #include "fake_llm_executor.h"
 #include "hip_llm_executor.h"
 #include "litertlm_reader.h"
+#include "model_file.h"
 #include "pipeline.h"
 #include "stop_token_detector.h"
 
@@ -374,6 +375,45 @@ int GiveBytes(const Status& s, std::string& bytes, uint8_t** data, uint64_t* len
 extern "C" {
 
 // The header of a .litertlm file (path != null) or of a buffer, as JSON text (malloc'd).
+// The section map and token capacity an executor takes from a model file: *json receives
+// {"sections": {"<kind>": [begin, end], ...}, "metadata_max_num_tokens": n, "max_num_tokens": what the settings end up with
+// when they arrive holding `preset_max_num_tokens` (0 = not set)}.
+int hle_model_file(const char* path, int32_t preset_max_num_tokens, char** json, char** err) {
+  auto file = LitertLmModelFile::Open(path);
+  if (!file.ok()) return Finish(file.status(), err);
+  auto from_metadata = file->MetadataMaxNumTokens();
+  if (!from_metadata.ok()) return Finish(from_metadata.status(), err);
+  auto settings = LlmExecutorSettings::CreateDefault(Backend::GPU_HIP);
+  if (!settings.ok()) return Finish(settings.status(), err);
+  settings->SetMaxNumTokens(preset_max_num_tokens);
+  Status s = file->UpdateExecutorSettings(&*settings);
+  if (!s.ok()) return Finish(s, err);
+  std::ostringstream os;
+  os << "{\"sections\": {";
+  bool first = true;
+  auto put = [&](const std::string& name, const std::optional<SectionRange>& r) {
+    if (!r.has_value()) return;
+    os << (first ? "" : ", ") << "\"" << name << "\": [" << r->begin << ", " << r->end << "]";
+    first = false;
+  };
+  for (ModelType t : {ModelType::kTfLitePrefillDecode, ModelType::kTfLiteEmbedder, ModelType::kTfLitePerLayerEmbedder,
+                      ModelType::kTfLiteAux})
+    put(ModelTypeToString(t), file->GetTFLiteModel(t));
+  put("SP_Tokenizer", file->GetSentencePieceTokenizer());
+  put("HF_Tokenizer_Zlib", file->GetHuggingFaceTokenizer());
+  put("LlmMetadataProto", file->GetLlmMetadata());
+  os << "}, \"metadata_max_num_tokens\": " << *from_metadata << ", \"max_num_tokens\": " << settings->GetMaxNumTokens() << "}";
+  *json = CopyText(os.str());
+  return 0;
+}
+// int32 varint field of a serialized protocol buffer; *value receives it (0 if absent).
+int hle_proto_int32_field(const void* data, uint64_t length, int32_t field_number, int32_t* value, char** err) {
+  auto r = ReadProtoInt32Field(std::string(static_cast<const char*>(data), static_cast<size_t>(length)), field_number);
+  if (!r.ok()) return Finish(r.status(), err);
+  *value = *r;
+  return 0;
+}
+
 int hle_litertlm_header(const char* path, const void* data, uint64_t length, char** json, char** err) {
   schema::LitertlmHeader header;
   Status s = path ? schema::ReadHeaderFromLiteRTLM(std::string(path), &header)

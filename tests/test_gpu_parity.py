@@ -580,7 +580,7 @@ def test_prefill_key_split_by_rule_softcap_and_limits():
 
 @ROWS16
 @pytest.mark.parametrize("dt", [A.F16, A.BF16])
-@pytest.mark.parametrize("hq,hkv,key_split", [(4, 1, 0), (8, 4, 0), (3, 1, 0), (4, 1, 3), (8, 4, 2)])
+@pytest.mark.parametrize("hq,hkv,key_split", [(4, 1, 0), (8, 4, 0), (3, 1, 0), (4, 1, 3), (8, 4, 2), (4, 1, 1)])
 def test_prefill_many_work_items_per_workgroup(dt, hq, hkv, key_split, rows16):
     """Few persistent workgroups walking many work items each (what one launch over 26 layers does on
     the full chip): the hand-over between items -- tickets, rings, query rows, output rows or parts of
