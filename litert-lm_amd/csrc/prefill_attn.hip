@@ -629,6 +629,7 @@ constexpr int kWaves16 = 4;
 constexpr int kRows16 = 16;
 constexpr int kSub16 = 2;       // sub-tiles of 16 query positions per wave
 constexpr int kKStages16 = 3, kVStages16 = 2;
+constexpr float kNoKeyYet = -1e30f;  // running reference of a query that has not met a visible key yet
 // LDS operand reads in flight ahead of their MFMAs, scores and P.V (four each would not fit in 256 registers)
 constexpr int kOpAhead = 3;
 constexpr int kOpAheadV = 3;
@@ -800,7 +801,7 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       for (int i = 0; i < NL; ++i) acc[u][i] = f4{0.f, 0.f, 0.f, 0.f};
     float m_run[kSub16], l_run[kSub16];
 #pragma unroll
-    for (int u = 0; u < kSub16; ++u) { m_run[u] = -INFINITY; l_run[u] = 0.f; }
+    for (int u = 0; u < kSub16; ++u) { m_run[u] = kNoKeyYet; l_run[u] = 0.f; }
     const int window = it.window, my_pos0 = it.my_pos0;
     const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
     const int wave_pos0 = __builtin_amdgcn_readfirstlane(my_pos0);
@@ -866,19 +867,27 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
           bm = wave_xor_max(bm, 32);
         }
         const float m_new = bm > m_run[u] + kRescaleSlack ? bm : m_run[u];
-        const float alpha = (m_run[u] == -INFINITY) ? 1.f : fast_exp2(m_run[u] - m_new);
-        const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
+        // (the reference starts at a finite kNoKeyYet, not at -inf: exp2(m_run - m_new) is then 0 when the first
+        // visible key arrives and 1 while none has, with no special cases; masked scores are -inf, so they weigh 0
+        // against either)
+        const float alpha = fast_exp2(m_run[u] - m_new);
+        const float neg_m = -m_new;
         m_run[u] = m_new;
         float lsum = 0.f;
         {
 #pragma unroll
           for (int T = 0; T < 2; ++T)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float pv = fast_exp2(fmaf(sc[u][T][e], c, neg_m));
-              p_hi[u][4 * T + e] = (_Float16)pv;
-              lsum += pv;
-            }
+            for (int e = 0; e < 4; ++e) p_hi[u][4 * T + e] = (_Float16)fast_exp2(fmaf(sc[u][T][e], c, neg_m));
+          // the row sum is taken over the probabilities as P.V will see them (rounded to half), two per
+          // instruction, accumulated in float32
+          using h2 = __attribute__((ext_vector_type(2))) _Float16;
+          const h2 ones = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            const h2 pair = {p_hi[u][2 * w], p_hi[u][2 * w + 1]};
+            lsum = __builtin_amdgcn_fdot2(pair, ones, lsum, false);
+          }
         }
         l_run[u] = l_run[u] * alpha + lsum;
         if (__any(alpha != 1.f)) {
