@@ -844,21 +844,37 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       // score sc[u][T][e]: key key0 + 16 T + 4 g + e against query my_pos0 + 16 u + n
       const int key0 = (it.kb0 + i) * kKeysPerBlock;
       const bool all_vis = key0 + kKeysPerBlock - 1 <= wave_pos0 && (unsigned)(wave_pos0 + kStretch - 1 - key0) < wlim;
+      if constexpr (CAP) {
+#pragma unroll
+        for (int u = 0; u < kSub16; ++u)
+#pragma unroll
+          for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sc[u][T][e] = (softcap * kLog2e) * fast_tanh(sc[u][T][e] * (a.scale / softcap));
+      }
+      if (!all_vis) {
+        // Only the block on the diagonal and the one at the window's edge hold keys that some query of the wave
+        // does not see. (A branch of its own: as part of the loop below the compiler turns the test into
+        // selects that every block pays for, 35 of ~130 vector-ALU instructions.)
+        asm volatile("; block with masked keys" ::: "memory");
+#pragma unroll
+        for (int u = 0; u < kSub16; ++u) {
+          const int my_pos = my_pos0 + kRows16 * u + n;
+#pragma unroll
+          for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              sc[u][T][e] = (unsigned)(my_pos - (key0 + 16 * T + 4 * g + e)) < wlim ? sc[u][T][e] : -INFINITY;
+        }
+      }
       h8 p_hi[kSub16];
 #pragma unroll
       for (int u = 0; u < kSub16; ++u) {
-        const int my_pos = my_pos0 + kRows16 * u + n;
         float bm = -INFINITY;
 #pragma unroll
         for (int T = 0; T < 2; ++T)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float x = sc[u][T][e];
-            if constexpr (CAP) x = (softcap * kLog2e) * fast_tanh(x * (a.scale / softcap));
-            if (!all_vis) x = (unsigned)(my_pos - (key0 + 16 * T + 4 * g + e)) < wlim ? x : -INFINITY;
-            sc[u][T][e] = x;
-            bm = fmaxf(bm, x);
-          }
+          for (int e = 0; e < 4; ++e) bm = fmaxf(bm, sc[u][T][e]);
         bm *= c;
         // The four lanes of a query compare notes only when one of them has seen a score that
         // exceeds the reference by more than the slack: rare after the first blocks.
