@@ -632,7 +632,7 @@ constexpr int kKStages16 = 3, kVStages16 = 2;
 constexpr float kNoKeyYet = -1e30f;  // running reference of a query that has not met a visible key yet
 // LDS operand reads in flight ahead of their MFMAs, scores and P.V (four each would not fit in 256 registers)
 constexpr int kOpAhead = 3;
-constexpr int kOpAheadV = 3;
+constexpr int kOpAheadV = 4;
 
 template <int D>
 constexpr int prefill16_lds_bytes() { return (kKStages16 + kVStages16) * 64 * D; }  // 80 KiB: two workgroups fill a CU's LDS
