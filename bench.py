@@ -381,7 +381,7 @@ def bench_pre_attention(A, torch, steps, warmup, layers=26, n=1024, hq=4, hkv=1)
             "single_token_latency_us": lat * 1e6}
 
 
-def pipeline_report(X, device_resident):
+def pipeline_report(X, device_resident, two_call_decode_step=False):
     """The reference's benchmark protocol (1024 prefill ids, 256 decode steps, README.md:390-400 of the
     reference) through the C++ executor, reported by the reference's own BenchmarkInfo text. The layers
     around attention are synthetic stand-ins; the rates say how the protocol runs end to end, they are
@@ -389,7 +389,7 @@ def pipeline_report(X, device_resident):
     import re
     layers = 26
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
-    kw = {"device_resident": bool(device_resident)}
+    kw = {"device_resident": bool(device_resident), "two_call_decode_step": bool(two_call_decode_step)}
     with X.HipLlmExecutor(layers, 4, 1, 64, 2048, runner_lengths=(1024,), layer_window=windows, fp16=True,
                           pre_attention=True, **kw) as ex:
         r = X.run_benchmark(ex, [3, 1, 4, 1, 5, 9, 2, 6], 1024, 256)
@@ -593,11 +593,16 @@ def main():
                              "fused step before attention), in the reference's report format; the layers other than "
                              "attention are synthetic stand-ins, so these are protocol figures, not kernel figures. "
                              "device_resident: activations, cache, logits and sampling stay on the GPU and only the "
-                             "token id returns; host_staged: float32 host tensors staged through the boundary per call"}
-            for mode, resident in (("device_resident", True), ("host_staged", False)):
+                             "token id returns, and a decode step makes one attention call per layer (mi355_attn_decode_step); "
+                             "device_resident_two_calls_per_layer: the same with mi355_attn_pre_attention and "
+                             "mi355_attn_decode as two calls; host_staged: float32 host tensors staged through the "
+                             "boundary per call"}
+            for mode, resident, two_calls in (("device_resident", True, False),
+                                              ("device_resident_two_calls_per_layer", True, True),
+                                              ("host_staged", False, False)):
                 if resident and not getattr(X, "HAS_DEVICE_RESIDENT", False):
                     continue
-                text, pre_tps, dec_tps = pipeline_report(X, resident)
+                text, pre_tps, dec_tps = pipeline_report(X, resident, two_calls)
                 log(f"[bench] the reference's benchmark protocol (1024 prefill / 256 decode ids), {mode}:\n" + text)
                 proto[mode] = {"prefill_tokens_per_s": pre_tps, "decode_tokens_per_s": dec_tps}
             lat = protocol_layer_latency(A, torch)

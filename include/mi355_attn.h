@@ -216,6 +216,26 @@ int mi355_attn_decode_layers(mi355_attn* handle, int32_t layer_begin, int32_t n_
                              void* out, int32_t num_splits, char** error_msg);
 
 /*
+ * One decode step of one layer in one launch: mi355_attn_pre_attention for the
+ * one new token of each of `batch` sequences (its row is kv_lens[b] - 1) and
+ * mi355_attn_decode over rows [0, kv_lens[b]). q [batch][num_q_heads][head_dim],
+ * k, v [batch][num_kv_heads][head_dim] are the raw projections (io_dtype); the
+ * normed / rotated key and value rows end up in the cache as
+ * mi355_attn_pre_attention leaves them, and `out` holds, bit for bit, what the
+ * two calls produce. Rows [0, kv_lens[b] - 1) must have been appended; the
+ * sequences of one call must differ; at most 64 sequences per call
+ * (kUnimplemented beyond: call in groups).
+ * Replaces: one layer's share of compiled_model_.Run("decode", ...)
+ * (llm_litert_compiled_model_executor.cc:407,522: cache update and attention
+ * are one graph invocation there) and, in the NPU flow, its RoPE, cache-update
+ * and attention signatures in turn
+ * (llm_litert_npu_compiled_model_executor.cc:1337-1530).
+ */
+int mi355_attn_decode_step(mi355_attn* handle, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,
+                           int32_t batch, const void* q, const void* k, const void* v, void* out,
+                           int32_t num_splits, char** error_msg);
+
+/*
  * mi355_attn_decode for callers that cannot allocate: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc. It has no
  * counterpart in the reference. Same arguments, same kernels and bit-identical

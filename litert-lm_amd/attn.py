@@ -91,6 +91,7 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_prefill_layers.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, errp]
     L.mi355_attn_decode.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
     L.mi355_attn_decode_noalloc.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
+    L.mi355_attn_decode_step.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, vp, vp, i32, errp]
     L.mi355_attn_decode_layers.argtypes = [vp, i32, i32, i32p, i32p, i32, vp, vp, i32, errp]
     L.mi355_attn_reset.argtypes = [vp, i32, errp]
     L.mi355_attn_sync.argtypes = [vp, errp]
@@ -244,6 +245,16 @@ class Attn:
             rc = lib().mi355_attn_decode_layers(self._h, layer, n_layers, sids, lens, batch, _ptr(q), _ptr(out),
                                                 num_splits, ctypes.byref(err))
         _check(rc, err)
+
+    def decode_step(self, layer, kv_lens, q, k, v, out, seq_ids=None, num_splits=0, batch=None):
+        """mi355_attn_decode_step: the step before attention for each sequence's one new token (row
+        kv_lens[b] - 1; q, k, v are the raw projections) and decode attention, in one launch."""
+        lens = kv_lens if isinstance(kv_lens, ctypes.Array) else _i32_array(kv_lens)
+        sids = seq_ids if isinstance(seq_ids, ctypes.Array) or seq_ids is None else _i32_array(seq_ids)
+        batch = len(lens) if batch is None else batch
+        err = ctypes.c_void_p()
+        _check(lib().mi355_attn_decode_step(self._h, layer, sids, lens, batch, _ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                            num_splits, ctypes.byref(err)), err)
 
     def decode_noalloc(self, layer, kv_lens, q, out, seq_ids=None, num_splits=0, batch=None):
         """mi355_attn_decode_noalloc: one layer, partials in the library's fixed workspace, no allocation."""

@@ -110,6 +110,16 @@ struct DecodeArgs {
   int32_t min_kv_len;        // min over kv_lens (host computed; only the launch rules look at it)
   float scale;               // softmax scale
   float softcap;
+  // The step before attention, run by the decode kernel itself for the one new token of every sequence
+  // (one layer, inline_items != 0): raw projections [batch][hq][D] / [batch][hkv][D] in the io dtype; the
+  // token's row is kv_len - 1. q is then unused. pre_q == nullptr: off. Flags and constants as in
+  // PreAttentionArgs.
+  const void* pre_q;
+  const void* pre_k;
+  const void* pre_v;
+  const float* pre_constants;
+  int32_t pre_rope, pre_norm_q, pre_norm_k, pre_norm_v, pre_q_scaled, pre_k_scaled;
+  float pre_eps, pre_weight_offset;
 };
 
 // Tokens per split-KV partition for a layer with the given window: the same

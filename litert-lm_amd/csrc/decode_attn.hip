@@ -24,6 +24,7 @@
 #include <hip/hip_ext.h>
 
 #include "mfma_util.h"
+#include "pre_attn_rows.h"
 
 namespace mi355 {
 namespace {
@@ -76,15 +77,17 @@ __device__ __forceinline__ void load_plane_block(u4 (&r)[D / 16], __amdgpu_buffe
 // n >= group are zero columns. A lane only ever reads the entries it wrote
 // itself, so no barrier is needed; keeping Q out of the register file leaves
 // room for two waves per SIMD next to the 128 registers of K/V data in flight.
+// q_rows: the `group` query rows of this KV head, [group][D] (in HBM, or in LDS when the kernel has
+// produced them itself).
 template <int KV, int IO, int D>
-__device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, int item, int kvh, int seq, int layer,
-                                        int lane) {
+__device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, const typename IoT<IO>::type* q_rows, int kvh,
+                                        int seq, int layer, int lane) {
   using io_t = typename IoT<IO>::type;
   constexpr int EPC = KvT<KV>::EPC;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   const int n = lane & 15, g = lane >> 4;
   const bool live = n < a.group;
-  const io_t* qrow = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group + (live ? n : 0)) * D;
+  const io_t* qrow = q_rows + (live ? n : 0) * D;
 #pragma unroll
   for (int step = 0; step < NQ; ++step) {
     u4 w;
@@ -184,10 +187,12 @@ __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)
 // reference max (exp2 domain), this lane's share of the sum (lane (n, g): head n,
 // tokens 4 g .. 4 g + 3 of every 16) and the unnormalised accumulators (channels
 // 16 * db + 4 * g .. + 3 of head n). Keys outside [vlo, p_hi) are masked.
-template <int KV, int IO, int D>
+// stage() leaves the Q operands in sm_q; it runs once the loads of the first block are under way.
+// hold_blk: a block whose rows stage() itself writes (-1: none); its loads are issued after stage().
+template <int KV, int IO, int D, class Stage>
 __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buffer_rsrc_t krsrc,
                                               __amdgpu_buffer_rsrc_t vrsrc, int first, int blk_end, int step, int vlo,
-                                              int p_hi, u4* sm_q, int item, int kvh, int seq, int layer, int lane,
+                                              int p_hi, const u4* sm_q, int hold_blk, Stage&& stage, int lane,
                                               float& m_run, float& l_run, f4 (&acc)[D / 16]) {
   constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
   constexpr int kBlockBytes = 64 * D;
@@ -198,11 +203,16 @@ __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buff
   // 16 to 32 KiB per wave are in flight while it computes.
   u4 kreg[NL], vreg[NL];
   int blk = __builtin_amdgcn_readfirstlane(first);
-  if (blk < blk_end) {
+  const bool early = blk < blk_end && blk != hold_blk;
+  if (early) {
     load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
     load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
   }
-  stage_q<KV, IO, D>(sm_q, a, item, kvh, seq, layer, lane);
+  stage();
+  if (blk < blk_end && !early) {
+    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
+    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
+  }
 
   m_run = -INFINITY;
   l_run = 0.f;
@@ -360,8 +370,17 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
 // the block index only. (With both sources behind one `cond ? a.inline_x[b] :
 // a.x[b]` the compiler selects a pointer and issues vector loads, one after the
 // other, and a wave spent 2 to 4 us before its first K/V load.)
-template <int KV, int IO, int D, int NW, bool INL>
+//
+// PRE (with INL, one layer): the kernel runs the step before attention for the one new token of its
+// sequence itself (row kv_len - 1): every workgroup norms and rotates the query rows of its KV head
+// into LDS; the workgroup whose partition ends at kv_len also norms / rotates the key and value rows
+// and writes them into the cache planes, waits until the stores have been acknowledged (s_waitcnt
+// vmcnt(0) in every wave, then the workgroup's barrier) and only then loads the block that holds
+// them: write and read go through the same CU and the same L2, and no other workgroup reads that
+// block (partitions are whole blocks). Same arithmetic, lane for lane, as pre_attention_kernel.
+template <int KV, int IO, int D, int NW, bool INL, bool PRE>
 __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
+  static_assert(!PRE || INL, "the fused step needs the items in the argument block");
   constexpr int VB = KvT<KV>::VB, NL = D / 16;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   extern __shared__ float smem[];
@@ -420,13 +439,66 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   u4* sm_q = reinterpret_cast<u4*>(smem) + wave * (NQ * 64);
   float m_run, l_run;
   f4 acc[NL];
-  stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, item, kvh, seq, layer, lane, m_run,
-                           l_run, acc);
+  using io_t = typename IoT<IO>::type;
+  if constexpr (PRE) {
+    static_assert(D == kRowD, "row helpers are written for head_dim 256");
+    const int G = a.group;
+    io_t* sm_rows = reinterpret_cast<io_t*>(smem + NW * NQ * 64 * 4 + NW * G * (D + 2));  // [G][D], behind the merge area
+    const int t = kv_len - 1;
+    const bool owns_row = p_hi == kv_len;  // exactly one partition per sequence and KV head
+    auto stage = [&]() {
+      const int nrows = G + (owns_row ? 2 : 0);  // G query rows, then the key and the value row
+      constexpr int kMaxRows = (kMaxGroup + 2 + NW - 1) / NW;
+      const int d0 = 2 * lane, d1 = D / 2 + 2 * lane;
+      float xs[kMaxRows][4];
+      // every row of this wave in flight before the first is waited for
+#pragma unroll
+      for (int r = 0; r < kMaxRows; ++r) {
+        const int row = wave + r * NW;
+        if (row < nrows) {
+          const void* src = row < G ? a.pre_q : (row == G ? a.pre_k : a.pre_v);
+          const int64_t base = row < G ? ((int64_t)b * a.hq + kvh * G + row) * D : ((int64_t)b * hkv + kvh) * D;
+          load_pair<IO>(src, base + d0, xs[r][0], xs[r][1]);
+          load_pair<IO>(src, base + d1, xs[r][2], xs[r][3]);
+        }
+      }
+      const RowAngles ang = row_angles(a.pre_rope ? a.pre_constants : nullptr, t, lane);
+#pragma unroll
+      for (int r = 0; r < kMaxRows; ++r) {
+        const int row = wave + r * NW;
+        if (row < nrows) {
+          const int kind = row < G ? 0 : (row == G ? 1 : 2);
+          const bool norm = kind == 0 ? a.pre_norm_q != 0 : (kind == 1 ? a.pre_norm_k != 0 : a.pre_norm_v != 0);
+          transform_row(xs[r], norm, row_weights(a.pre_constants, kind, a.pre_q_scaled != 0, a.pre_k_scaled != 0),
+                        a.pre_weight_offset, a.pre_eps, a.pre_rope != 0 && kind != 2, ang, lane);
+          if (kind == 0) {
+            uint8_t* dst = reinterpret_cast<uint8_t*>(sm_rows + row * D);
+            store_pair<IO>(dst + d0 * sizeof(io_t), xs[r][0], xs[r][1]);
+            store_pair<IO>(dst + d1 * sizeof(io_t), xs[r][2], xs[r][3]);
+          } else {
+            const int is_v = kind - 1;
+            uint8_t* plane = const_cast<uint8_t*>(kplane) + is_v * plane_bytes;
+            const float* sc = KV == kI8 ? a.scales + a.geom.scale_offset(layer, seq, is_v, kvh) : nullptr;
+            store_cache_row<KV>(plane, sc, is_v, t, xs[r], lane);
+          }
+        }
+      }
+      if (owns_row) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the new rows have reached L2
+      __syncthreads();
+      stage_q<KV, IO, D>(sm_q, a, sm_rows, kvh, seq, layer, lane);
+    };
+    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, owns_row ? t / VB : -1, stage,
+                             lane, m_run, l_run, acc);
+  } else {
+    const io_t* q_rows = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group) * D;
+    auto stage = [&]() { stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane); };
+    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, -1, stage, lane, m_run, l_run,
+                             acc);
+  }
   float l_tot = wave_xor_add(l_run, 16);
   l_tot = wave_xor_add(l_tot, 32);
 
   const int G = a.group;
-  using io_t = typename IoT<IO>::type;
   if constexpr (NW == 1) {
     // One wave: nothing to merge. Lane (n, g) holds channels 16 * db + 4 * g .. + 3 of head n.
     if (n < G) {
@@ -502,14 +574,15 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   }
 }
 
-template <int KV, int IO, int D, int NW, bool INL>
+template <int KV, int IO, int D, int NW, bool INL, bool PRE = false>
 hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const dim3 grid(a.n_layers, a.batch, a.num_splits * a.geom.hkv);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
-  const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float);
+  const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float) +
+                     (PRE ? (size_t)a.group * D * sizeof(typename IoT<IO>::type) : 0);
   // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
   // begin and end timestamps, not the host-side launch latency around it.
-  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
+  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL, PRE>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || a.num_splits == 1) return err;
   hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D, INL>), dim3(a.hq, a.batch, a.n_layers), dim3(D), 0, stream, a);
@@ -518,6 +591,10 @@ hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, h
 
 template <int KV, int IO, int D, int NW>
 hipError_t launch_variant(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  if (a.pre_q) {
+    if (!a.inline_items || a.n_layers != 1) return hipErrorInvalidValue;
+    return launch_inl<KV, IO, D, NW, true, true>(a, stream, ev0, ev1);
+  }
   if (a.inline_items && a.n_layers <= kInlineLayers) return launch_inl<KV, IO, D, NW, true>(a, stream, ev0, ev1);
   return launch_inl<KV, IO, D, NW, false>(a, stream, ev0, ev1);
 }

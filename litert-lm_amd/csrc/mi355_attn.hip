@@ -244,11 +244,29 @@ void fill_inline_windows(const mi355_attn* h, DecodeArgs* a) {
   for (int i = 0; i < a->n_layers; ++i) a->inline_window[i] = h->window[a->layer_begin + i];
 }
 
+// Raw projections of the one new token of every sequence (mi355_attn_decode_step): the decode kernel runs the
+// step before attention itself.
+struct NewRows {
+  const void* k;
+  const void* v;
+};
+
 // no_alloc: the call may not allocate (mi355_attn_decode_noalloc): device pointers only, and the
 // partials go to this GPU's `scratch` instead of the handle's growable workspace.
+// new_rows: q holds raw query projections and the new token's key / value rows come with the call
+// (its row, kv_lens[b] - 1, need not have been appended).
 int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq_ids, const int32_t* kv_lens,
-                int batch, const void* q, void* out, int num_splits, char** error_msg, bool no_alloc = false) {
+                int batch, const void* q, void* out, int num_splits, char** error_msg, bool no_alloc = false,
+                const NewRows* new_rows = nullptr) {
   if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (new_rows) {
+    if (!new_rows->k || !new_rows->v) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null k or v");
+    if (batch > kInlineItems)
+      return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
+                  "mi355_attn_decode_step takes up to %d sequences per call (got %d): call it in groups, or "
+                  "mi355_attn_pre_attention per sequence and mi355_attn_decode",
+                  kInlineItems, batch);
+  }
   if (no_alloc && h->cfg.host_io)
     return fail(error_msg, MI355_ATTN_FAILED_PRECONDITION,
                 "mi355_attn_decode_noalloc needs device pointers (the handle was created with host_io = 1, "
@@ -275,10 +293,15 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
       return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "kv_lens[%d]=%d outside [1, max_tokens=%d]", b, len,
                   h->cfg.max_tokens);
     for (int l = layer_begin; l < layer_begin + n_layers; ++l)
-      if (len > h->filled[(size_t)l * h->cfg.max_seqs + seq])
+      if (len - (new_rows ? 1 : 0) > h->filled[(size_t)l * h->cfg.max_seqs + seq])
         return fail(error_msg, MI355_ATTN_OUT_OF_RANGE,
                     "kv_lens[%d]=%d but only %d rows of layer %d, sequence %d were appended", b, len,
                     h->filled[(size_t)l * h->cfg.max_seqs + seq], l, seq);
+    if (new_rows)  // every sequence gets one new row: the same sequence twice would write two
+      for (int c = 0; c < b; ++c)
+        if ((seq_ids ? seq_ids[c] : c) == seq)
+          return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq_ids[%d] and seq_ids[%d] name the same sequence %d", c,
+                      b, seq);
     max_len = std::max(max_len, len);
     min_len = std::min(min_len, len);
   }
@@ -320,6 +343,22 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   const void* dq = nullptr;
   void* dout = nullptr;
   if (int rc = stage_in(h, 0, q, io_bytes, &dq, error_msg)) return rc;
+  if (new_rows) {
+    const size_t kv_bytes = (size_t)batch * h->cfg.num_kv_heads * h->cfg.head_dim * io_size(h);
+    if (int rc = stage_in(h, 2, new_rows->k, kv_bytes, &a.pre_k, error_msg)) return rc;
+    if (int rc = stage_in(h, 3, new_rows->v, kv_bytes, &a.pre_v, error_msg)) return rc;
+    a.pre_q = dq;
+    const mi355_attn::LayerTransform& lt = h->transform[layer_begin];  // never set: a plain append
+    a.pre_constants = h->d_transform + (size_t)layer_begin * transform_floats(h->cfg.head_dim);
+    a.pre_rope = lt.rope;
+    a.pre_norm_q = lt.norm_q;
+    a.pre_norm_k = lt.norm_k;
+    a.pre_norm_v = lt.norm_v;
+    a.pre_q_scaled = lt.q_scaled;
+    a.pre_k_scaled = lt.k_scaled;
+    a.pre_eps = lt.eps;
+    a.pre_weight_offset = lt.weight_offset;
+  }
   if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
   if (batch <= kInlineItems) {
     a.inline_items = 1;
@@ -348,6 +387,8 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream,
                               h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr));
   h->timed = h->timing;
+  if (new_rows)
+    for (int b = 0; b < batch; ++b) note_rows_written(h, layer_begin, seq_ids ? seq_ids[b] : b, kv_lens[b] - 1, 1);
   return stage_out_end(h, 1, out, io_bytes, error_msg);
 }
 
@@ -813,6 +854,13 @@ int mi355_attn_decode_layers(mi355_attn* h, int32_t layer_begin, int32_t n_layer
                              const int32_t* kv_lens, int32_t batch, const void* q, void* out, int32_t num_splits,
                              char** error_msg) {
   return decode_impl(h, layer_begin, n_layers, seq_ids, kv_lens, batch, q, out, num_splits, error_msg);
+}
+
+int mi355_attn_decode_step(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens, int32_t batch,
+                           const void* q, const void* k, const void* v, void* out, int32_t num_splits,
+                           char** error_msg) {
+  const NewRows rows{k, v};
+  return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg, /*no_alloc=*/false, &rows);
 }
 
 int mi355_attn_decode_noalloc(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,

@@ -32,6 +32,7 @@ class _Config(ctypes.Structure):
         ("num_runners", ctypes.c_int32), ("fp16_activations", ctypes.c_int32),
         ("recording_backend", ctypes.c_int32), ("execute_pending_on_single_id_chunk", ctypes.c_int32),
         ("softcap", ctypes.c_float), ("pre_attention", ctypes.c_int32), ("device_resident", ctypes.c_int32),
+        ("two_call_decode_step", ctypes.c_int32),
     ]
 
 
@@ -110,16 +111,17 @@ class HipLlmExecutor:
 
     def __init__(self, num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens, runner_lengths=(1024,),
                  layer_window=None, fp16=False, recording_backend=False, execute_pending_on_single_id_chunk=False,
-                 softcap=0.0, pre_attention=False, device_resident=None):
+                 softcap=0.0, pre_attention=False, device_resident=None, two_call_decode_step=False):
         """device_resident: True / False, or None to let the executor decide (device-resident on its own MI355X
-        backend, host-staged on the recording backend)."""
+        backend, host-staged on the recording backend). two_call_decode_step: device-resident decode keeps the step
+        before attention and the attention as two calls per layer instead of one (comparisons)."""
         self._win = _arr(layer_window) if layer_window is not None else None
         self._runners = _arr(runner_lengths)
         cfg = _Config(num_layers, num_q_heads, num_kv_heads, vocab, max_num_tokens,
                       ctypes.cast(self._win, ctypes.POINTER(ctypes.c_int32)) if self._win is not None else None,
                       ctypes.cast(self._runners, ctypes.POINTER(ctypes.c_int32)), len(runner_lengths), int(fp16),
                       int(recording_backend), int(execute_pending_on_single_id_chunk), softcap, int(pre_attention),
-                      -1 if device_resident is None else int(bool(device_resident)))
+                      -1 if device_resident is None else int(bool(device_resident)), int(bool(two_call_decode_step)))
         self._h = ctypes.c_void_p()
         err = ctypes.c_void_p()
         _check(lib().hle_create(ctypes.byref(cfg), ctypes.byref(self._h), ctypes.byref(err)), err)

@@ -68,6 +68,13 @@ class AttentionBackend {
   virtual Status PreAttentionOnDevice(int, int, int, void*, const void*, const void*) { return NotDeviceResident(); }
   virtual Status PrefillOnDevice(int, int, int, const void*, void*) { return NotDeviceResident(); }
   virtual Status DecodeOnDevice(int, int, const void*, void*) { return NotDeviceResident(); }
+  // PreAttentionOnDevice for the one row at kv_len - 1 and DecodeOnDevice in one queued call (same results); q, k, v
+  // are the raw projections of that row. A backend without such a call answers kUnimplemented and the executor
+  // makes the two calls.
+  virtual Status DecodeStepOnDevice(int, int, const void*, const void*, const void*, void*) {
+    return UnimplementedError("attention backend '" + Name() + "' has no single-call decode step.");
+  }
+  virtual bool HasDecodeStep() const { return false; }
   virtual Status Sync() { return OkStatus(); }  // waits for everything queued on Stream()
 
  protected:

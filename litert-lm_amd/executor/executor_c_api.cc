@@ -50,6 +50,7 @@ struct hle_config {
   float softcap;
   int32_t pre_attention;             // 1: the layers hand over raw projections; Gemma-3-like norm + rotary constants
   int32_t device_resident;           // -1: the executor decides, 0: host-staged, 1: device-resident
+  int32_t two_call_decode_step;      // 1: device-resident decode keeps pre-attention and attention as two calls per layer
 };
 
 int hle_create(const hle_config* c, void** out, char** err) {
@@ -73,6 +74,7 @@ int hle_create(const hle_config* c, void** out, char** err) {
   options.residency = c->device_resident < 0    ? HipExecutorOptions::Residency::kAuto
                       : c->device_resident == 0 ? HipExecutorOptions::Residency::kHost
                                                 : HipExecutorOptions::Residency::kDevice;
+  options.single_call_decode_step = c->two_call_decode_step == 0;
   std::unique_ptr<AttentionBackend> backend;
   if (c->recording_backend) backend = std::make_unique<RecordingAttentionBackend>(shape);
   auto ex = HipLlmExecutor::Create(*settings, std::make_unique<SyntheticDecoderLayers>(shape, c->vocab), options,

@@ -341,7 +341,15 @@ Status HipLlmExecutor::RunTokensOnDevice(const std::vector<int32_t>& tokens, con
   RETURN_IF_ERROR(HipStatus(hipSetDevice(device_->device), "hipSetDevice"));
   const DecoderLayers::DeviceActivations& io = device_->io;
   RETURN_IF_ERROR(layers_->BeginOnDevice(tokens, positions, io));
+  // One-token passes over layers with a transform: the step before attention and the attention in one launch.
+  const bool single_call_step = options_.single_call_decode_step && is_decode && n == 1 && !shape.transforms.empty() &&
+                                backend_->HasDecodeStep();
   for (int layer = 0; layer < shape.num_layers; ++layer) {
+    if (single_call_step) {
+      RETURN_IF_ERROR(backend_->DecodeStepOnDevice(layer, pos0 + 1, io.q, io.k, io.v, io.attn));
+      RETURN_IF_ERROR(layers_->NextLayerOnDevice(layer, io));
+      continue;
+    }
     if (shape.transforms.empty()) {
       RETURN_IF_ERROR(backend_->AppendOnDevice(layer, pos0, n, io.k, io.v));
     } else {

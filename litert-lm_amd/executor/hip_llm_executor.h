@@ -40,6 +40,10 @@ struct HipExecutorOptions {
   // per call. kAuto: kDevice when the decoder layers have a device form and no backend was injected, else kHost.
   enum class Residency { kAuto, kHost, kDevice };
   Residency residency = Residency::kAuto;
+  // Device-resident one-token passes over layers with a transform: true (default) queues the step before
+  // attention and the attention as one call per layer where the backend has one (same results); false keeps
+  // the two calls (comparisons).
+  bool single_call_decode_step = true;
 };
 
 // One forward pass as the executor issued it (kept for tests and debugging).

@@ -52,6 +52,13 @@ class Mi355AttentionBackend : public AttentionBackend {
     const int32_t len = kv_len;
     return FromCode(mi355_attn_decode(h_, layer, nullptr, &len, 1, q, out, 0, &err), err, "decode");
   }
+  bool HasDecodeStep() const override { return device_resident_; }
+  Status DecodeStepOnDevice(int layer, int kv_len, const void* q, const void* k, const void* v, void* out) override {
+    if (!device_resident_) return NotDeviceResident();
+    char* err = nullptr;
+    const int32_t len = kv_len;
+    return FromCode(mi355_attn_decode_step(h_, layer, nullptr, &len, 1, q, k, v, out, 0, &err), err, "decode_step");
+  }
   Status Sync() override {
     char* err = nullptr;
     return FromCode(mi355_attn_sync(h_, &err), err, "sync");
