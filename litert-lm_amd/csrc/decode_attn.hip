@@ -188,12 +188,13 @@ __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)
 // tokens 4 g .. 4 g + 3 of every 16) and the unnormalised accumulators (channels
 // 16 * db + 4 * g .. + 3 of head n). Keys outside [vlo, p_hi) are masked.
 // stage() leaves the Q operands in sm_q; it runs once the loads of the first block are under way.
-// hold_blk: a block whose rows stage() itself writes (-1: none); its loads are issued after stage().
-template <int KV, int IO, int D, class Stage>
+// patch_blk: a block one of whose rows is not in the cache yet (-1: none); patch(kreg, vreg) puts that
+// row into the block's registers once they are loaded.
+template <int KV, int IO, int D, class Stage, class Patch>
 __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buffer_rsrc_t krsrc,
                                               __amdgpu_buffer_rsrc_t vrsrc, int first, int blk_end, int step, int vlo,
-                                              int p_hi, const u4* sm_q, int hold_blk, Stage&& stage, int lane,
-                                              float& m_run, float& l_run, f4 (&acc)[D / 16]) {
+                                              int p_hi, const u4* sm_q, int patch_blk, Stage&& stage, Patch&& patch,
+                                              int lane, float& m_run, float& l_run, f4 (&acc)[D / 16]) {
   constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
   constexpr int kBlockBytes = 64 * D;
   const int g = lane >> 4;
@@ -203,16 +204,11 @@ __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buff
   // 16 to 32 KiB per wave are in flight while it computes.
   u4 kreg[NL], vreg[NL];
   int blk = __builtin_amdgcn_readfirstlane(first);
-  const bool early = blk < blk_end && blk != hold_blk;
-  if (early) {
+  if (blk < blk_end) {
     load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
     load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
   }
   stage();
-  if (blk < blk_end && !early) {
-    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
-    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
-  }
 
   m_run = -INFINITY;
   l_run = 0.f;
@@ -225,6 +221,7 @@ __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buff
     // they would occupy 32 to 64 registers for the whole kernel.
     int qi = lane;
     asm volatile("" : "+v"(qi));
+    if (blk == patch_blk) patch(kreg, vreg);
     f4 s[NT];
     qk_block<KV, D>(kreg, sm_q, qi, s);
     const int nxt = blk + step;
@@ -372,12 +369,15 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
 // other, and a wave spent 2 to 4 us before its first K/V load.)
 //
 // PRE (with INL, one layer): the kernel runs the step before attention for the one new token of its
-// sequence itself (row kv_len - 1): every workgroup norms and rotates the query rows of its KV head
-// into LDS; the workgroup whose partition ends at kv_len also norms / rotates the key and value rows
-// and writes them into the cache planes, waits until the stores have been acknowledged (s_waitcnt
-// vmcnt(0) in every wave, then the workgroup's barrier) and only then loads the block that holds
-// them: write and read go through the same CU and the same L2, and no other workgroup reads that
-// block (partitions are whole blocks). Same arithmetic, lane for lane, as pre_attention_kernel.
+// sequence itself (row t = kv_len - 1): every workgroup norms and rotates the query rows of its KV
+// head into LDS; the workgroup whose partition ends at kv_len also norms / rotates the key and value
+// rows, stores them into the cache planes for later calls, and keeps them in LDS in the planes' element
+// format: the wave that streams the block of row t loads it like any other block (the row's bytes are
+// stale, or change under the load) and overwrites the row's bytes in its registers from LDS before the
+// block is used. The MFMAs see the operands that a load after pre_attention_kernel would have
+// delivered, so the results are the same bit for bit, and nothing waits for a store. No other
+// workgroup reads that block (partitions are whole blocks). Same arithmetic, lane for lane, as
+// pre_attention_kernel.
 template <int KV, int IO, int D, int NW, bool INL, bool PRE>
 __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
   static_assert(!PRE || INL, "the fused step needs the items in the argument block");
@@ -442,8 +442,13 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
   using io_t = typename IoT<IO>::type;
   if constexpr (PRE) {
     static_assert(D == kRowD, "row helpers are written for head_dim 256");
+    constexpr int ESZ = KV == kF32 ? 4 : (KV == kI8 ? 1 : 2);
+    constexpr int NT = VB / 16, KPT = NL / NT;
     const int G = a.group;
-    io_t* sm_rows = reinterpret_cast<io_t*>(smem + NW * NQ * 64 * 4 + NW * G * (D + 2));  // [G][D], behind the merge area
+    // behind the merge area: [G][D] query rows (io type), then the new key and value row as the planes hold them
+    io_t* sm_rows = reinterpret_cast<io_t*>(smem + NW * NQ * 64 * 4 + NW * G * (D + 2));
+    uint8_t* sm_krow = reinterpret_cast<uint8_t*>(sm_rows + G * D);
+    uint8_t* sm_vrow = sm_krow + D * ESZ;
     const int t = kv_len - 1;
     const bool owns_row = p_hi == kv_len;  // exactly one partition per sequence and KV head
     auto stage = [&]() {
@@ -479,21 +484,57 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
             const int is_v = kind - 1;
             uint8_t* plane = const_cast<uint8_t*>(kplane) + is_v * plane_bytes;
             const float* sc = KV == kI8 ? a.scales + a.geom.scale_offset(layer, seq, is_v, kvh) : nullptr;
-            store_cache_row<KV>(plane, sc, is_v, t, xs[r], lane);
+            store_cache_row<KV, false>(plane, sc, is_v, t, xs[r], lane);
+            store_cache_row<KV, true>(is_v ? sm_vrow : sm_krow, sc, is_v, t, xs[r], lane);
           }
         }
       }
-      if (owns_row) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the new rows have reached L2
       __syncthreads();
       stage_q<KV, IO, D>(sm_q, a, sm_rows, kvh, seq, layer, lane);
     };
+    // Row t in the registers of its block. K: chunk c of the row is the 16 bytes of lane (t % 16, g) in load
+    // (t % VB) / 16 * KPT + j with c = 4 j + g. V: element d of the row sits in lane (d % 16, (t % 16) / 4), load
+    // d / 16, at element slot 4 * ((t % VB) / 16) + t % 4 of the lane's 16 bytes.
+    auto patch = [&](u4 (&kreg)[NL], u4 (&vreg)[NL]) {
+      const int tb = t % VB;
+      const int tile = tb >> 4;
+      const bool k_lane = (lane & 15) == (tb & 15);
+#pragma unroll
+      for (int T = 0; T < NT; ++T) {
+        if (T == tile) {
+#pragma unroll
+          for (int j = 0; j < KPT; ++j) {
+            const u4 fresh = *reinterpret_cast<const u4*>(sm_krow + (4 * j + g) * 16);
+            kreg[T * KPT + j] = k_lane ? fresh : kreg[T * KPT + j];
+          }
+        }
+      }
+      const int byte0 = (4 * tile + (tb & 3)) * ESZ;  // of the lane's 16 bytes
+      const unsigned in_word = ESZ == 4 ? 0xffffffffu : ((ESZ == 2 ? 0xffffu : 0xffu) << (8 * (byte0 & 3)));
+      const bool v_lane = g == ((tb & 15) >> 2);
+      unsigned mask[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) mask[w] = (v_lane && w == (byte0 >> 2)) ? in_word : 0u;
+#pragma unroll
+      for (int db = 0; db < NL; ++db) {
+        const uint8_t* src = sm_vrow + (16 * db + n) * ESZ;
+        unsigned e;
+        if constexpr (ESZ == 4) e = *reinterpret_cast<const unsigned*>(src);
+        else if constexpr (ESZ == 2) e = *reinterpret_cast<const uint16_t*>(src);
+        else e = *src;
+        e <<= 8 * (byte0 & 3);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) vreg[db][w] = (vreg[db][w] & ~mask[w]) | (e & mask[w]);
+      }
+    };
     stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, owns_row ? t / VB : -1, stage,
-                             lane, m_run, l_run, acc);
+                             patch, lane, m_run, l_run, acc);
   } else {
     const io_t* q_rows = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group) * D;
     auto stage = [&]() { stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane); };
-    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, -1, stage, lane, m_run, l_run,
-                             acc);
+    auto patch = [](u4 (&)[NL], u4 (&)[NL]) {};
+    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, -1, stage, patch, lane, m_run,
+                             l_run, acc);
   }
   float l_tot = wave_xor_add(l_run, 16);
   l_tot = wave_xor_add(l_tot, 32);
@@ -579,7 +620,7 @@ hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, h
   const dim3 grid(a.n_layers, a.batch, a.num_splits * a.geom.hkv);
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   const size_t lds = (size_t)NW * NQ * 64 * 16 + (size_t)NW * a.group * (D + 2) * sizeof(float) +
-                     (PRE ? (size_t)a.group * D * sizeof(typename IoT<IO>::type) : 0);
+                     (PRE ? (size_t)a.group * D * sizeof(typename IoT<IO>::type) + 2 * (size_t)D * a.geom.esize : 0);
   // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
   // begin and end timestamps, not the host-side launch latency around it.
   hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL, PRE>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
@@ -619,6 +660,8 @@ hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t 
     // 4096 tokens: 6.5 instead of 6.1 TB/s; sequences of equal length lose 1 % and keep one wave).
     if (a.num_splits == 1 && wgs >= 1024 && a.min_kv_len * 4 < a.max_kv_len * 3) waves = 4;
   }
+  // The fused step before attention is serial work per wave (group + 2 rows): at least two waves share it.
+  if (a.pre_q && t.waves == 0 && waves == 1) waves = 2;
   if (waves == 1) return launch_variant<KV, IO, D, 1>(a, s, e0, e1);
   if (waves == 2) return launch_variant<KV, IO, D, 2>(a, s, e0, e1);
   return launch_variant<KV, IO, D, 4>(a, s, e0, e1);

@@ -132,13 +132,20 @@ __device__ __forceinline__ const float* row_weights(const float* constants, int 
 }
 
 // The transformed key (is_v 0) or value (is_v 1) row of token t into its plane; `scales` = the plane's
-// [256] dequantisation scales (int8 cache only).
-template <int KV>
+// [256] dequantisation scales (int8 cache only). LINEAR: `plane` is a buffer of 256 elements instead and
+// element d of the row goes to element d of the buffer, in the same element format.
+template <int KV, bool LINEAR = false>
 __device__ __forceinline__ void store_cache_row(uint8_t* plane, const float* scales, int is_v, int t,
                                                 const float (&x)[4], int lane) {
   constexpr int ESZ = KV == kF32 ? 4 : (KV == kI8 ? 1 : 2);
   constexpr int EPC = 16 / ESZ;
   const int d0 = 2 * lane, d1 = kRowD / 2 + 2 * lane;
+  auto k_chunk_offset = [](int tt, int c, int, int) -> int64_t {
+    return LINEAR ? (int64_t)c * 16 : mi355::k_chunk_offset(tt, c, kRowD, ESZ);
+  };
+  auto v_elem_offset = [](int tt, int d, int, int) -> int64_t {
+    return LINEAR ? (int64_t)d * ESZ : mi355::v_elem_offset(tt, d, kRowD, ESZ);
+  };
   if constexpr (KV == kI8) {
     const float2 s0 = *reinterpret_cast<const float2*>(scales + d0);
     const float2 s1 = *reinterpret_cast<const float2*>(scales + d1);
