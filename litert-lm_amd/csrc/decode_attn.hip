@@ -378,9 +378,16 @@ __global__ void __launch_bounds__(D) decode_merge_kernel(const DecodeArgs a) {
 // delivered, so the results are the same bit for bit, and nothing waits for a store. No other
 // workgroup reads that block (partitions are whole blocks). Same arithmetic, lane for lane, as
 // pre_attention_kernel.
+// The rows are serial work for a wave (a norm with its cross-lane sums per row, two full-precision
+// sincosf per lane), so a PRE workgroup always has four waves to share them; those beyond NW leave
+// after the rows, and the attention itself runs on NW waves exactly as without PRE.
+template <int NW, bool PRE>
+constexpr int decode_wg_waves() { return PRE && NW < 4 ? 4 : NW; }
+
 template <int KV, int IO, int D, int NW, bool INL, bool PRE>
-__global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArgs a) {
+__global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_attn_kernel(const DecodeArgs a) {
   static_assert(!PRE || INL, "the fused step needs the items in the argument block");
+  constexpr int NWP = decode_wg_waves<NW, PRE>();  // waves of the workgroup; the first NW do the attention
   constexpr int VB = KvT<KV>::VB, NL = D / 16;
   constexpr int NQ = KV == kF32 ? D / 16 : D / 32;
   extern __shared__ float smem[];
@@ -451,15 +458,15 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
     uint8_t* sm_vrow = sm_krow + D * ESZ;
     const int t = kv_len - 1;
     const bool owns_row = p_hi == kv_len;  // exactly one partition per sequence and KV head
-    auto stage = [&]() {
+    auto rows = [&]() __attribute__((always_inline)) {
       const int nrows = G + (owns_row ? 2 : 0);  // G query rows, then the key and the value row
-      constexpr int kMaxRows = (kMaxGroup + 2 + NW - 1) / NW;
+      constexpr int kMaxRows = (kMaxGroup + 2 + NWP - 1) / NWP;
       const int d0 = 2 * lane, d1 = D / 2 + 2 * lane;
       float xs[kMaxRows][4];
       // every row of this wave in flight before the first is waited for
 #pragma unroll
       for (int r = 0; r < kMaxRows; ++r) {
-        const int row = wave + r * NW;
+        const int row = wave + r * NWP;
         if (row < nrows) {
           const void* src = row < G ? a.pre_q : (row == G ? a.pre_k : a.pre_v);
           const int64_t base = row < G ? ((int64_t)b * a.hq + kvh * G + row) * D : ((int64_t)b * hkv + kvh) * D;
@@ -470,7 +477,7 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
       const RowAngles ang = row_angles(a.pre_rope ? a.pre_constants : nullptr, t, lane);
 #pragma unroll
       for (int r = 0; r < kMaxRows; ++r) {
-        const int row = wave + r * NW;
+        const int row = wave + r * NWP;
         if (row < nrows) {
           const int kind = row < G ? 0 : (row == G ? 1 : 2);
           const bool norm = kind == 0 ? a.pre_norm_q != 0 : (kind == 1 ? a.pre_norm_k != 0 : a.pre_norm_v != 0);
@@ -490,12 +497,19 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
         }
       }
       __syncthreads();
+    };
+    if (wave >= NW) {  // a helper wave: its share of the rows, nothing else
+      rows();
+      return;
+    }
+    auto stage = [&]() __attribute__((always_inline)) {
+      rows();
       stage_q<KV, IO, D>(sm_q, a, sm_rows, kvh, seq, layer, lane);
     };
     // Row t in the registers of its block. K: chunk c of the row is the 16 bytes of lane (t % 16, g) in load
     // (t % VB) / 16 * KPT + j with c = 4 j + g. V: element d of the row sits in lane (d % 16, (t % 16) / 4), load
     // d / 16, at element slot 4 * ((t % VB) / 16) + t % 4 of the lane's 16 bytes.
-    auto patch = [&](u4 (&kreg)[NL], u4 (&vreg)[NL]) {
+    auto patch = [&](u4 (&kreg)[NL], u4 (&vreg)[NL]) __attribute__((always_inline)) {
       const int tb = t % VB;
       const int tile = tb >> 4;
       const bool k_lane = (lane & 15) == (tb & 15);
@@ -531,7 +545,7 @@ __global__ void __launch_bounds__(NW * 64, 2) decode_attn_kernel(const DecodeArg
                              patch, lane, m_run, l_run, acc);
   } else {
     const io_t* q_rows = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group) * D;
-    auto stage = [&]() { stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane); };
+    auto stage = [&]() __attribute__((always_inline)) { stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane); };
     auto patch = [](u4 (&)[NL], u4 (&)[NL]) {};
     stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, -1, stage, patch, lane, m_run,
                              l_run, acc);
@@ -623,7 +637,8 @@ hipError_t launch_inl(const DecodeArgs& a, hipStream_t stream, hipEvent_t ev0, h
                      (PRE ? (size_t)a.group * D * sizeof(typename IoT<IO>::type) + 2 * (size_t)D * a.geom.esize : 0);
   // ev0/ev1 are attached to the dispatch itself: they carry the kernel's own
   // begin and end timestamps, not the host-side launch latency around it.
-  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL, PRE>), grid, dim3(NW * 64), lds, stream, ev0, ev1, 0, a);
+  hipExtLaunchKernelGGL((decode_attn_kernel<KV, IO, D, NW, INL, PRE>), grid, dim3(decode_wg_waves<NW, PRE>() * 64), lds,
+                        stream, ev0, ev1, 0, a);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess || a.num_splits == 1) return err;
   hipLaunchKernelGGL((decode_merge_kernel<KV, IO, D, INL>), dim3(a.hq, a.batch, a.n_layers), dim3(D), 0, stream, a);
@@ -660,8 +675,6 @@ hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t 
     // 4096 tokens: 6.5 instead of 6.1 TB/s; sequences of equal length lose 1 % and keep one wave).
     if (a.num_splits == 1 && wgs >= 1024 && a.min_kv_len * 4 < a.max_kv_len * 3) waves = 4;
   }
-  // The fused step before attention is serial work per wave (group + 2 rows): at least two waves share it.
-  if (a.pre_q && t.waves == 0 && waves == 1) waves = 2;
   if (waves == 1) return launch_variant<KV, IO, D, 1>(a, s, e0, e1);
   if (waves == 2) return launch_variant<KV, IO, D, 2>(a, s, e0, e1);
   return launch_variant<KV, IO, D, 4>(a, s, e0, e1);

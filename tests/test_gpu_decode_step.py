@@ -138,6 +138,13 @@ def test_full_batch_of_64():
     drive_both(A.F16, 4, 1, lens, 2, [0], 0, 0, seed=5)
 
 
+@pytest.mark.parametrize("kv", [A.F16, A.BF16, A.I8])
+def test_long_context(kv):
+    say(f"decode_step kv {kv}: context 4090 -> 4096, positions where the angles are thousands of radians")
+    drive_both(kv, 8, 2, [4090], 6, [0, 512], 0, 0, seed=6)
+    drive_both(kv, 8, 2, [4090, 2047], 2, [0], 16, 0, seed=7)
+
+
 def test_against_the_oracles():
     """Rows and attention of one fused step against the CPU oracles (fp16, window 64)."""
     n, hq, hkv, dt = 200, 4, 1, A.F16
