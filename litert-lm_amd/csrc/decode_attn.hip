@@ -458,6 +458,8 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
     uint8_t* sm_vrow = sm_krow + D * ESZ;
     const int t = kv_len - 1;
     const bool owns_row = p_hi == kv_len;  // exactly one partition per sequence and KV head
+    // (always_inline: called from two places, the lambda was compiled as a function otherwise, and a sixteenth of
+    // the outputs came out wrong)
     auto rows = [&]() __attribute__((always_inline)) {
       const int nrows = G + (owns_row ? 2 : 0);  // G query rows, then the key and the value row
       constexpr int kMaxRows = (kMaxGroup + 2 + NWP - 1) / NWP;
