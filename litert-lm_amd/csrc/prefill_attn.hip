@@ -1092,7 +1092,62 @@ int tile_key_blocks(const PrefillArgs& a, int rows_per_tile, int w, int t) {
 // costs about 3 us besides its blocks (start, store). Both workgroups of a compute unit should finish together:
 // a workgroup left alone runs faster (1.5 us per block) but the compute unit as a whole slower than the pair.
 // With one workgroup per compute unit or fewer, all workgroups are alike.
+//
+// Launches of two workgroups per compute unit with up to kPackMaxItems items are packed instead (pack_by_deadline):
+// longest first is a poor packer when most items are of one size (config 2: 356 of 832 items are 17 key blocks
+// for 512 workgroups, and the items of 9 to 16 blocks end up on top of a 17 instead of on top of each other).
 constexpr long kPlanMaxItems = 1L << 22;
+constexpr size_t kPackMaxItems = 4096;
+
+// Best fit, decreasing, under a deadline found by bisection: every item (longest first) goes to the workgroup
+// that it fills up best without passing the deadline - of its layer's home XCD if one there can take it, else
+// of any. The clock is a least-squares fit of the lifetimes of the 512 workgroups of the measured launch
+// (times in units of 0.05 us): a first-placed workgroup 8.1 us + 1.4 us per key block, a second-placed one
+// 7.05 us + 2.2 us per block (it is served second whenever both want the same pipe), 5 us per item.
+// blocks[i], home_xcd[i]: key blocks and home XCD of item i (items sorted by blocks, longest first).
+// Returns false when nothing was packed (never with the bounds of the bisection below).
+bool pack_by_deadline(const std::vector<int32_t>& blocks, const std::vector<int>& home_xcd, int wgs, int cus, int xcds,
+                      std::vector<int>* owner) {
+  constexpr long kFirstStart = 162, kFirstBlock = 28, kSecondStart = 141, kSecondBlock = 44, kItem = 100;
+  auto done_at = [&](int g, long blk, long cnt) {
+    return g < cus ? kFirstStart + kFirstBlock * blk + kItem * cnt : kSecondStart + kSecondBlock * blk + kItem * cnt;
+  };
+  std::vector<long> blk(wgs), cnt(wgs);
+  auto attempt = [&](long deadline, std::vector<int>* out) {
+    std::fill(blk.begin(), blk.end(), 0L);
+    std::fill(cnt.begin(), cnt.end(), 0L);
+    for (size_t i = 0; i < blocks.size(); ++i) {
+      int pick = -1;
+      long pick_done = -1;
+      for (int pass = 0; pass < 2 && pick < 0; ++pass) {
+        if (pass == 1 && xcds <= 1) break;
+        for (int g = 0; g < wgs; ++g) {
+          if (pass == 0 && xcds > 1 && g % xcds != home_xcd[i]) continue;
+          const long t = done_at(g, blk[g] + blocks[i], cnt[g] + 1);
+          if (t <= deadline && t > pick_done) {
+            pick_done = t;
+            pick = g;
+          }
+        }
+      }
+      if (pick < 0) return false;
+      blk[pick] += blocks[i];
+      ++cnt[pick];
+      if (out) (*out)[i] = pick;
+    }
+    return true;
+  };
+  long total = 0;
+  for (int32_t b : blocks) total += b;
+  long lo = 0, hi = kFirstStart + kSecondStart + kSecondBlock * total + kItem * (long)blocks.size();  // one workgroup takes all
+  while (hi - lo > 4) {
+    const long mid = (lo + hi) / 2;
+    if (attempt(mid, nullptr)) hi = mid;
+    else lo = mid;
+  }
+  return attempt(hi, owner);
+}
+
 void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::vector<int32_t>* words) {
   const int rows_per_tile = kStretch * (4 / hpb);
   const int tiles = (a.n + rows_per_tile - 1) / rows_per_tile;
@@ -1135,6 +1190,20 @@ void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::ve
       xcd_work[x] += layer_work[li];
     }
   }
+  std::vector<int> owner(items.size());
+  std::vector<int> count(wgs, 0);
+  bool packed = false;
+  if (paired && items.size() <= kPackMaxItems) {
+    std::vector<int32_t> blocks(items.size());
+    std::vector<int> home_xcd(items.size());
+    for (size_t i = 0; i < items.size(); ++i) {
+      blocks[i] = items[i].blocks;
+      home_xcd[i] = home[items[i].unit / per_layer];
+    }
+    packed = pack_by_deadline(blocks, home_xcd, wgs, cus, xcds, &owner);
+    if (packed)
+      for (size_t i = 0; i < items.size(); ++i) ++count[owner[i]];
+  }
   // (time done, workgroup) min-heaps per XCD: the first-placed workgroups and the second-placed ones
   using Entry = std::pair<long, int>;
   auto later = [](const Entry& x, const Entry& y) { return x > y; };
@@ -1147,9 +1216,7 @@ void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::ve
     std::make_heap(first[x].begin(), first[x].end(), later);
     std::make_heap(second[x].begin(), second[x].end(), later);
   }
-  std::vector<int> owner(items.size());
-  std::vector<int> count(wgs, 0);
-  for (size_t i = 0; i < items.size(); ++i) {
+  for (size_t i = 0; i < items.size() && !packed; ++i) {
     // the best workgroup of an XCD for this item: (time it would be done, which heap)
     auto best_of = [&](int x) {
       long t = -1;
