@@ -7,6 +7,8 @@ generated code never touches them except as MFMA operands: a copy or a spill pla
 them before the data has arrived. This script reads the device assembly (hipcc -S) and fails if, in any
 instantiation of the kernel, an instruction other than an MFMA names one of those registers after the first load.
 
+It also fails when an instantiation spills vector registers.
+
     check_query_registers.py prefill_attn.s
 """
 import re
@@ -46,9 +48,15 @@ def main(path):
             if registers(m.group(2)) & query:
                 print(f"{name}: line {i}: `{line.strip()}` touches a query register")
                 bad += 1
+    # No instantiation may spill vector registers: the loop is laid out for exactly 256 of them, and a spill is
+    # scratch traffic plus a wait inside every key block (it has happened after changes that looked harmless).
+    for name, count in re.findall(r"\.name:\s+(_ZN5mi355\w*prefill_attn16_kernel\w+)\s.*?\.vgpr_spill_count:\s+(\d+)", asm, re.S):
+        if int(count):
+            print(f"{name}: {count} vector registers spilled")
+            bad += 1
     if bad:
         sys.exit(1)
-    print(f"{path}: query registers of {len(kernels)} kernel instantiations are touched by MFMAs only")
+    print(f"{path}: query registers of {len(kernels)} kernel instantiations are touched by MFMAs only, no vector register spills")
 
 
 if __name__ == "__main__":
