@@ -35,6 +35,7 @@
 #include <utility>
 
 #include <algorithm>
+#include <set>
 #include <vector>
 
 #include "attn_params.h"
@@ -1093,7 +1094,8 @@ int tile_key_blocks(const PrefillArgs& a, int rows_per_tile, int w, int t) {
 // a workgroup left alone runs faster (1.5 us per block) but the compute unit as a whole slower than the pair.
 // With one workgroup per compute unit or fewer, all workgroups are alike.
 //
-// Launches of two workgroups per compute unit with up to kPackMaxItems items are packed instead (pack_by_deadline):
+// Launches over several layers, of two workgroups per compute unit and up to kPackMaxItems items, are packed instead
+// (pack_by_deadline):
 // longest first is a poor packer when most items are of one size (config 2: 356 of 832 items are 17 key blocks
 // for 512 workgroups, and the items of 9 to 16 blocks end up on top of a 17 instead of on top of each other).
 constexpr long kPlanMaxItems = 1L << 22;
@@ -1108,38 +1110,50 @@ constexpr size_t kPackMaxItems = 4096;
 // Returns false when nothing was packed (never with the bounds of the bisection below).
 bool pack_by_deadline(const std::vector<int32_t>& blocks, const std::vector<int>& home_xcd, int wgs, int cus, int xcds,
                       std::vector<int>* owner) {
-  constexpr long kFirstStart = 162, kFirstBlock = 28, kSecondStart = 141, kSecondBlock = 44, kItem = 100;
-  auto done_at = [&](int g, long blk, long cnt) {
-    return g < cus ? kFirstStart + kFirstBlock * blk + kItem * cnt : kSecondStart + kSecondBlock * blk + kItem * cnt;
-  };
-  std::vector<long> blk(wgs), cnt(wgs);
+  constexpr long kStart[2] = {162, 141}, kBlock[2] = {28, 44}, kItem = 100;  // [0] first-placed, [1] second-placed
+  // The workgroups of an XCD and a kind, ordered by the time they are done: the best fit for an item is the
+  // last one that still meets the deadline with it (a search in the ordered set, not a scan of all workgroups:
+  // a plan is built whenever a launch shape is new, and a scan costs milliseconds).
+  using Slot = std::pair<long, int>;  // (time done, workgroup)
+  std::vector<std::set<Slot>> sets((size_t)xcds * 2);
   auto attempt = [&](long deadline, std::vector<int>* out) {
-    std::fill(blk.begin(), blk.end(), 0L);
-    std::fill(cnt.begin(), cnt.end(), 0L);
+    for (auto& s : sets) s.clear();
+    for (int g = 0; g < wgs; ++g) {
+      const int kind = g < cus ? 0 : 1;
+      sets[(size_t)(g % xcds) * 2 + kind].insert({kStart[kind], g});
+    }
     for (size_t i = 0; i < blocks.size(); ++i) {
-      int pick = -1;
+      std::set<Slot>* pick_set = nullptr;
+      std::set<Slot>::iterator pick_it;
       long pick_done = -1;
-      for (int pass = 0; pass < 2 && pick < 0; ++pass) {
-        if (pass == 1 && xcds <= 1) break;
-        for (int g = 0; g < wgs; ++g) {
-          if (pass == 0 && xcds > 1 && g % xcds != home_xcd[i]) continue;
-          const long t = done_at(g, blk[g] + blocks[i], cnt[g] + 1);
-          if (t <= deadline && t > pick_done) {
-            pick_done = t;
-            pick = g;
+      auto look = [&](int x) {
+        for (int kind = 0; kind < 2; ++kind) {
+          std::set<Slot>& s = sets[(size_t)x * 2 + kind];
+          const long cost = kBlock[kind] * blocks[i] + kItem;
+          auto it = s.upper_bound({deadline - cost, INT32_MAX});
+          if (it == s.begin()) continue;
+          --it;
+          if (it->first + cost > pick_done) {
+            pick_done = it->first + cost;
+            pick_set = &s;
+            pick_it = it;
           }
         }
-      }
-      if (pick < 0) return false;
-      blk[pick] += blocks[i];
-      ++cnt[pick];
-      if (out) (*out)[i] = pick;
+      };
+      look(xcds > 1 ? home_xcd[i] : 0);
+      if (!pick_set)
+        for (int x = 0; x < xcds; ++x) look(x);
+      if (!pick_set) return false;
+      const int g = pick_it->second;
+      pick_set->erase(pick_it);
+      pick_set->insert({pick_done, g});
+      if (out) (*out)[i] = g;
     }
     return true;
   };
   long total = 0;
   for (int32_t b : blocks) total += b;
-  long lo = 0, hi = kFirstStart + kSecondStart + kSecondBlock * total + kItem * (long)blocks.size();  // one workgroup takes all
+  long lo = 0, hi = kStart[0] + kStart[1] + kBlock[1] * total + kItem * (long)blocks.size();  // one workgroup takes all
   while (hi - lo > 4) {
     const long mid = (lo + hi) / 2;
     if (attempt(mid, nullptr)) hi = mid;
@@ -1193,7 +1207,9 @@ void build_prefill_plan(const PrefillArgs& a, int hpb, int wgs, int cus, std::ve
   std::vector<int> owner(items.size());
   std::vector<int> count(wgs, 0);
   bool packed = false;
-  if (paired && items.size() <= kPackMaxItems) {
+  // (launches over several layers only: their shapes repeat, and the plan is kept; packing costs about a millisecond
+  // of host time per new shape, longest-first a tenth of that)
+  if (paired && a.n_layers > 1 && items.size() <= kPackMaxItems) {
     std::vector<int32_t> blocks(items.size());
     std::vector<int> home_xcd(items.size());
     for (size_t i = 0; i < items.size(); ++i) {
