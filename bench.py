@@ -411,6 +411,31 @@ def protocol_layer_latency(A, torch, ctx=1152):
     return sec
 
 
+def decode_step_latency(A, torch, ctx=1152):
+    """One decode step of one layer at the same shape from the raw projections of the new token (Gemma-3-like
+    norms and rotary embedding): mi355_attn_pre_attention + mi355_attn_decode (two calls) against
+    mi355_attn_decode_step (one call, the same bits). Seconds per step, (two calls, one call)."""
+    at = A.Attn(1, 4, 1, D, 2048, 1, A.F16, A.F16)
+    fill_cache(at, torch, 1, [ctx], 1, torch.float16, seed=7)
+    ones = np.ones(D, np.float32)
+    at.set_layer_transform(0, norm_q=True, norm_k=True, q_weight=ones, k_weight=ones, eps=1e-6,
+                           rope_inv_freq=(10000.0 ** (-np.arange(0, D, 2, dtype=np.float64) / D)).astype(np.float32))
+    q = torch.randn((1, 4, D), device="cuda:0").half()
+    k = torch.randn((1, 1, D), device="cuda:0").half()
+    v = torch.randn((1, 1, D), device="cuda:0").half()
+    q_rot, out = torch.empty_like(q), torch.empty_like(q)
+    lens = A._i32_array([ctx])
+
+    def two_calls(i):
+        at.pre_attention(0, 0, ctx - 1, q, k, v, q_rot)
+        at.decode(0, lens, q_rot, out, num_splits=0, batch=1)
+
+    two, _ = time_steps(torch, two_calls, 500, 50)
+    one, _ = time_steps(torch, lambda i: at.decode_step(0, lens, q, k, v, out, num_splits=0, batch=1), 500, 50)
+    at.close()
+    return two, one
+
+
 def cpu_baseline_c3(layers, ctx, budget_s=24.0):
     """C restatement of the reference CPU op order (fp32, OpenMP) on the same
     30-layer decode sweep, repeated until about `budget_s` seconds are spent:
@@ -607,6 +632,9 @@ def main():
                 proto[mode] = {"prefill_tokens_per_s": pre_tps, "decode_tokens_per_s": dec_tps}
             lat = protocol_layer_latency(A, torch)
             proto["one_layer_decode_attention_latency_us"] = round(lat * 1e6, 2)
+            two, one = decode_step_latency(A, torch)
+            proto["one_layer_decode_step_latency_us"] = {"pre_attention_then_decode": round(two * 1e6, 2),
+                                                         "decode_step": round(one * 1e6, 2)}
             proto["decode_tokens_per_s_if_only_attention_ran"] = round(1.0 / (26 * lat), 1)
             if "device_resident" in proto:
                 proto["device_resident_fraction_of_that"] = round(
