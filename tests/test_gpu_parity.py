@@ -807,6 +807,43 @@ def test_error_codes():
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("seed", [3, 8, 12])
+def test_prefill_launch_over_many_layers_random_shapes(seed):
+    """Launches over several layers on the kernel with host-planned work lists (two workgroups per CU, items
+    packed under a deadline): random layer counts, head groupings, windows, chunk positions and lengths. Every
+    output row must have been written (the buffer starts as NaN: an item the plan dropped would leave its rows),
+    and the result must agree with the other prefill kernel, which shares no scheduling code with it, to the
+    rounding of the output format (2e-3 fp16; bf16 outputs differ by up to one rounding step, 2^-8 of max|ref|)."""
+    rng = np.random.default_rng(seed)
+    layers = int(rng.integers(8, 40))
+    hq, hkv = [(4, 1), (8, 2), (2, 2), (16, 2)][int(rng.integers(0, 4))]
+    n = int(rng.integers(200, 1500))
+    pos0 = int(rng.integers(0, 3)) * int(rng.integers(0, 700))
+    windows = [int(rng.choice([0, 0, 64, 512, 100])) for _ in range(layers)]
+    dt = A.F16 if rng.random() < 0.5 else A.BF16
+    say(f"prefill over {layers} layers, Hq{hq}/Hkv{hkv}, rows [{pos0}, {pos0 + n}), dtype {dt}")
+    cap = pos0 + n
+    outs = []
+    for rows16 in (1, 0):
+        with make(layers, hq, hkv, cap, 1, dt, layer_window=windows) as at:
+            at.set_option("prefill_rows16", rows16)
+            g = torch.Generator(device=DEV).manual_seed(seed)
+            for layer in range(layers):
+                k = torch.randn((cap, hkv, D), generator=g, device=DEV).to(TDT[dt])
+                v = torch.randn((cap, hkv, D), generator=g, device=DEV).to(TDT[dt])
+                at.kv_append(layer, 0, 0, k, v)
+            q = torch.randn((layers, n, hq, D), generator=g, device=DEV).to(TDT[dt])
+            out = torch.full_like(q, float("nan"))
+            at.prefill(0, 0, pos0, n, q, out, n_layers=layers)
+            torch.cuda.synchronize()
+            outs.append(out.float())
+    assert torch.isfinite(outs[0]).all(), "rows left unwritten by the planned kernel"
+    assert torch.isfinite(outs[1]).all()
+    err = float((outs[0] - outs[1]).abs().max() / outs[1].abs().max())
+    say(f"  kernels differ by {err:.2e}")
+    assert err < (2e-3 if dt == A.F16 else 2.0 ** -8 + 2e-3)
+
+
 def test_host_io_mode():
     # host pointers at the boundary, as the reference's host TensorBuffers
     L = 130
