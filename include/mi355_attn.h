@@ -253,6 +253,19 @@ int mi355_attn_decode_noalloc(mi355_attn* handle, int32_t layer, const int32_t* 
                               int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg);
 
 /*
+ * Host only, no device needed (tests of the planner; no counterpart in the reference): the work plan that a
+ * prefill launch of n rows at q_pos0 over n_layers layers gets on `workgroups` workgroups of a part with
+ * `compute_units` compute units (the kernel on 16x16x32 MFMAs: which workgroup runs which (layer, head block,
+ * 32-position tile) items). items_per_wg / blocks_per_wg: [workgroups] out, the items and the key blocks of each
+ * workgroup; items_off_home (may be NULL): items placed on another XCD than most of their layer's.
+ * Returns the number of items (every item of the launch exactly once), < 0 on bad arguments or a broken plan.
+ */
+int mi355_attn_prefill_plan_probe(int32_t n_layers, int32_t n, int32_t q_pos0, int32_t num_q_heads,
+                                  int32_t num_kv_heads, const int32_t* layer_window, int32_t workgroups,
+                                  int32_t compute_units, int32_t* items_per_wg, int32_t* blocks_per_wg,
+                                  int32_t* items_off_home);
+
+/*
  * Forgets the rows of sequence `seq` (seq < 0: all). Like
  * LlmLiteRtCompiledModelExecutor::Reset
  * (llm_litert_compiled_model_executor.cc:568-574) the cache memory itself is

@@ -50,6 +50,13 @@ struct PrefillPlans {
 };
 void free_prefill_plans(PrefillPlans* plans);
 
+// Host only (no device is touched): the plan of a launch of n query rows at q_pos0 over n_layers layers on `wgs`
+// workgroups of a part with `cus` compute units. items_per_wg / blocks_per_wg: [wgs] out; items_off_home (may be
+// null): items that run on another XCD than most of their layer. Returns the number of items, -1 for bad
+// arguments, -2 when an item appears twice, -3 when one is missing.
+int prefill_plan_probe(int n_layers, int n, int q_pos0, int hq, int hkv, const int32_t* layer_window, int wgs, int cus,
+                       int32_t* items_per_wg, int32_t* blocks_per_wg, int32_t* items_off_home);
+
 // With args.kchunk > 0 the merge kernel follows the attention kernel (ev1 then marks the end of the
 // attention kernel alone).
 hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, PrefillPlans* plans,

@@ -856,6 +856,13 @@ int mi355_attn_decode_layers(mi355_attn* h, int32_t layer_begin, int32_t n_layer
   return decode_impl(h, layer_begin, n_layers, seq_ids, kv_lens, batch, q, out, num_splits, error_msg);
 }
 
+int mi355_attn_prefill_plan_probe(int32_t n_layers, int32_t n, int32_t q_pos0, int32_t num_q_heads, int32_t num_kv_heads,
+                                  const int32_t* layer_window, int32_t workgroups, int32_t compute_units,
+                                  int32_t* items_per_wg, int32_t* blocks_per_wg, int32_t* items_off_home) {
+  return mi355::prefill_plan_probe(n_layers, n, q_pos0, num_q_heads, num_kv_heads, layer_window, workgroups, compute_units,
+                                   items_per_wg, blocks_per_wg, items_off_home);
+}
+
 int mi355_attn_decode_step(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens, int32_t batch,
                            const void* q, const void* k, const void* v, void* out, int32_t num_splits,
                            char** error_msg) {

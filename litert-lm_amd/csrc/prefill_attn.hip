@@ -1416,6 +1416,62 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
 
 }  // namespace
 
+// Host only: the work plan of a launch shape without launching anything (tests of the planner).
+int prefill_plan_probe(int n_layers, int n, int q_pos0, int hq, int hkv, const int32_t* layer_window, int wgs, int cus,
+                       int32_t* items_per_wg, int32_t* blocks_per_wg, int32_t* items_off_home) {
+  if (n_layers < 1 || n < 1 || q_pos0 < 0 || hq < 1 || hkv < 1 || hq % hkv != 0 || wgs < 1 || cus < 0 || !layer_window ||
+      !items_per_wg || !blocks_per_wg)
+    return -1;
+  PrefillArgs a{};
+  a.n_layers = n_layers;
+  a.n = n;
+  a.q_pos0 = q_pos0;
+  a.hq = hq;
+  a.group = hq / hkv;
+  a.geom.hkv = hkv;
+  a.host_window = layer_window;
+  const int G = a.group;
+  const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
+  const int rows_per_tile = kStretch * (4 / hpb);
+  const int per_layer = hkv * (G / hpb);
+  std::vector<int32_t> words;
+  build_prefill_plan(a, hpb, wgs, cus, &words);
+  const int32_t* offs = words.data();
+  const int32_t* list = words.data() + wgs + 1;
+  const int total = offs[wgs];
+  // every (unit, tile) exactly once
+  std::set<std::pair<int32_t, int32_t>> seen;
+  for (int i = 0; i < total; ++i)
+    if (!seen.insert({list[2 * i], list[2 * i + 1]}).second) return -2;
+  const int tiles = (n + rows_per_tile - 1) / rows_per_tile;
+  if ((long)seen.size() != (long)n_layers * per_layer * tiles) return -3;
+  // the home XCD of a layer as the planner computes it is not recomputed here: a layer's home is taken to be the XCD
+  // that holds most of its items
+  constexpr int kXcds = 8;
+  std::vector<std::vector<int>> per_layer_xcd(n_layers, std::vector<int>(kXcds, 0));
+  for (int g = 0; g < wgs; ++g) {
+    items_per_wg[g] = offs[g + 1] - offs[g];
+    long blocks = 0;
+    for (int i = offs[g]; i < offs[g + 1]; ++i) {
+      const int li = list[2 * i] / per_layer, tile = list[2 * i + 1] & 0xFFFFF;
+      blocks += tile_key_blocks(a, rows_per_tile, layer_window[li], tile);
+      ++per_layer_xcd[li][g % kXcds];
+    }
+    blocks_per_wg[g] = (int32_t)blocks;
+  }
+  if (items_off_home) {
+    long off = 0;
+    for (int li = 0; li < n_layers; ++li) {
+      const auto& v = per_layer_xcd[li];
+      const int most = *std::max_element(v.begin(), v.end());
+      for (int x = 0; x < kXcds; ++x) off += v[x];
+      off -= most;
+    }
+    *items_off_home = (int32_t)off;
+  }
+  return total;
+}
+
 PrefillSplit plan_prefill_split(const PrefillArgs& a, int option) {
   PrefillSplit out;
   if (option == 0 || !a.host_window) return out;
