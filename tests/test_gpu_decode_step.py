@@ -173,6 +173,45 @@ def test_against_the_oracles():
         assert orc.rel_err(host(vo)[0], want_v[n - 1]) < 2e-3
 
 
+def test_replayed_from_a_hip_graph():
+    """Three layers' steps captured into one HIP graph (the calls allocate nothing once the split-KV workspace
+    exists) and replayed several times, with eager work and synchronisations in between: every replay leaves
+    what the eager calls left."""
+    hq, hkv, dt, n, layers = 8, 2, A.F16, 333, 3
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with A.Attn(layers, hq, hkv, D, 512, 1, dt, dt, layer_window=[0, 64, 0], stream=side.cuda_stream) as at:
+            for layer in range(layers):
+                at.set_layer_transform(layer, norm_q=True, norm_k=True, eps=1e-6,
+                                       rope_inv_freq=po.rope_inv_freq(D, 10000.0))
+                q0, k0, v0 = rows(31 + layer, dt, n - 1, hq, D), rows(41 + layer, dt, n - 1, hkv, D), rows(51 + layer, dt, n - 1, hkv, D)
+                at.pre_attention(layer, 0, 0, q0, k0, v0, torch.empty_like(q0))
+            q, k, v = rows(61, dt, layers, 1, hq, D), rows(62, dt, layers, 1, hkv, D), rows(63, dt, layers, 1, hkv, D)
+            out = torch.zeros_like(q)
+
+            def steps():
+                for layer in range(layers):
+                    at.decode_step(layer, [n], q[layer], k[layer], v[layer], out[layer])
+
+            steps()  # eager: the workspace is allocated here
+            side.synchronize()
+            want = out.clone()
+            assert torch.isfinite(want.float()).all() and want.float().abs().max() > 0
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                steps()
+            for replay in range(4):
+                out.zero_()
+                side.synchronize()
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(out, want), f"replay {replay}"
+                steps()  # eager work between the replays
+                side.synchronize()
+                assert torch.equal(out, want)
+            del graph
+
+
 def test_host_pointers():
     """A handle that stages host buffers (host_io = 1) gives the same step."""
     hq, hkv, dt, n = 4, 1, A.F16, 70
