@@ -15,9 +15,7 @@ i32 = ctypes.c_int32
 
 
 def lib():
-    if not os.path.exists(LIB):
-        pytest.skip("libmi355_attn.so not built")
-    L = ctypes.CDLL(LIB)
+    L = ctypes.CDLL(LIB)  # (a missing library is a failure, not a skip: the build comes first)
     L.mi355_attn_prefill_plan_probe.restype = ctypes.c_int
     return L
 
