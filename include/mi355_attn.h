@@ -21,6 +21,17 @@
  *   k, v   : [n][num_kv_heads][head_dim]         kv_dtype
  *   scales : [num_kv_heads][head_dim]            float32 (int8 cache only)
  * Query head h reads KV head h / (num_q_heads / num_kv_heads).
+ * Cache type and activation type (io_dtype: queries in, attention out) are set
+ * apart as the reference sets them apart (ActivationDataType,
+ * runtime/executor/executor_settings_base.h:54-66; its GPU path keeps an fp16
+ * cache under fp32 activations when asked,
+ * llm_litert_compiled_model_executor.cc:609-617). Pairs: io_dtype equal to
+ * kv_dtype (f32, f16, bf16); f32 activations over an f16 or bf16 cache; an
+ * int8 cache under f16, bf16 or f32 activations. The matrix cores take the
+ * queries in the cache's operand type: float32 queries over a 16-bit cache
+ * are rounded to it (nearest even) on the way in (a prefill call does so in a
+ * pass of its own over the query rows), products accumulate in float32 and
+ * the output is written in io_dtype from those sums.
  * A bfloat16 cache keeps its K planes in bfloat16 and its V planes as IEEE half
  * values, so that the probabilities multiply V with 11 significant bits on the
  * fp16 matrix-core path: a bfloat16 value v is stored without loss for
@@ -223,8 +234,9 @@ int mi355_attn_decode_layers(mi355_attn* handle, int32_t layer_begin, int32_t n_
  * normed / rotated key and value rows end up in the cache as
  * mi355_attn_pre_attention leaves them, and `out` holds, bit for bit, what the
  * two calls produce. Rows [0, kv_lens[b] - 1) must have been appended; the
- * sequences of one call must differ; at most 64 sequences per call
- * (kUnimplemented beyond: call in groups).
+ * sequences of one call must differ. A launch carries up to 64 sequences; a
+ * larger batch runs as several launches queued back to back (everything that
+ * can be refused is checked for the whole batch before the first).
  * Replaces: one layer's share of compiled_model_.Run("decode", ...)
  * (llm_litert_compiled_model_executor.cc:407,522: cache update and attention
  * are one graph invocation there) and, in the NPU flow, its RoPE, cache-update

@@ -104,8 +104,9 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_cache_bytes.argtypes = [vp]
     L.mi355_attn_cache_bytes.restype = ctypes.c_uint64
     L.mi355_attn_version.restype = ctypes.c_char_p
-    for name in ("create", "kv_append", "kv_set_scales", "kv_read", "prefill", "prefill_layers", "decode",
-                 "decode_layers", "decode_noalloc", "reset", "sync", "set_timing", "set_option"):
+    for name in ("create", "kv_append", "kv_set_scales", "kv_read", "set_layer_transform", "pre_attention", "prefill",
+                 "prefill_layers", "decode", "decode_layers", "decode_step", "decode_noalloc", "prefill_plan_probe",
+                 "reset", "sync", "set_timing", "set_option"):
         getattr(L, "mi355_attn_" + name).restype = c
     _lib = L
     return L

@@ -141,8 +141,9 @@ MI355_HD void decode_visible_range(int kv_len, int window, int* vlo, int* start)
 }
 
 struct PrefillArgs {
-  const void* q;   // [n_layers][n][hq][D]
+  const void* q;   // [n_layers][n][hq][D], io type
   void* out;
+  void* q_stage;   // float32 activations over a 16-bit cache: room for the queries in the cache's type (else unused)
   const uint8_t* cache;
   const float* scales;
   const int32_t* layer_window;

@@ -79,6 +79,32 @@ __device__ __forceinline__ void load_plane_block(u4 (&r)[D / 16], __amdgpu_buffe
 // room for two waves per SIMD next to the 128 registers of K/V data in flight.
 // q_rows: the `group` query rows of this KV head, [group][D] (in HBM, or in LDS when the kernel has
 // produced them itself).
+// Eight consecutive query elements of the io type as float32 (two vectors of four: plain values, no array
+// that could end up in scratch memory).
+struct Q8 { f4 lo, hi; };
+template <int IO>
+__device__ __forceinline__ Q8 load_q8(const typename IoT<IO>::type* p) {
+  Q8 r;
+  if constexpr (IO == kF32) {
+    r.lo = *reinterpret_cast<const f4*>(p);
+    r.hi = *reinterpret_cast<const f4*>(p + 4);
+  } else if constexpr (IO == kF16) {
+    const h8 v = *reinterpret_cast<const h8*>(p);
+    r.lo = f4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    r.hi = f4{(float)v[4], (float)v[5], (float)v[6], (float)v[7]};
+  } else {
+    const b8 v = *reinterpret_cast<const b8*>(p);
+    r.lo = f4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    r.hi = f4{(float)v[4], (float)v[5], (float)v[6], (float)v[7]};
+  }
+  return r;
+}
+
+// The activation type (IO: queries in, attention out) need not be the cache's: a 16-bit cache serves float32
+// activations (the reference's ActivationDataType::FLOAT32 over its fp16 GPU cache,
+// runtime/executor/executor_settings_base.h:54-66), an int8 cache any of the three. The matrix cores take
+// the queries in the cache's operand type, so float32 queries are rounded to it here (to nearest even), once
+// per call; the output is written in the io type from the float32 accumulators.
 template <int KV, int IO, int D>
 __device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, const typename IoT<IO>::type* q_rows, int kvh,
                                         int seq, int layer, int lane) {
@@ -92,16 +118,28 @@ __device__ __forceinline__ void stage_q(u4* sm_q, const DecodeArgs& a, const typ
   for (int step = 0; step < NQ; ++step) {
     u4 w;
     if constexpr (KV == kI8) {
-      static_assert(IO == kF16, "int8 cache pairs with fp16 queries");
       const float* ks = a.scales + a.geom.scale_offset(layer, seq, 0, kvh);
       const int d0 = (4 * (step >> 1) + g) * EPC + 8 * (step & 1);
-      const h8 qv = *reinterpret_cast<const h8*>(qrow + d0);
-      h8 o;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = (_Float16)((float)qv[e] * ks[d0 + e]);
+      const Q8 x = load_q8<IO>(qrow + d0);
+      const f4 s0 = *reinterpret_cast<const f4*>(ks + d0), s1 = *reinterpret_cast<const f4*>(ks + d0 + 4);
+      const f4 y0 = x.lo * s0, y1 = x.hi * s1;
+      const h8 o = {(_Float16)y0[0], (_Float16)y0[1], (_Float16)y0[2], (_Float16)y0[3],
+                    (_Float16)y1[0], (_Float16)y1[1], (_Float16)y1[2], (_Float16)y1[3]};
       w = bit_cast<u4>(o);
-    } else {
+    } else if constexpr (KV == IO) {
       w = *reinterpret_cast<const u4*>(qrow + (4 * step + g) * EPC);
+    } else {
+      static_assert(IO == kF32 && (KV == kF16 || KV == kBF16), "float32 activations over a 16-bit cache");
+      const Q8 x = load_q8<IO>(qrow + (4 * step + g) * EPC);
+      if constexpr (KV == kF16) {
+        const h8 o = {(_Float16)x.lo[0], (_Float16)x.lo[1], (_Float16)x.lo[2], (_Float16)x.lo[3],
+                      (_Float16)x.hi[0], (_Float16)x.hi[1], (_Float16)x.hi[2], (_Float16)x.hi[3]};
+        w = bit_cast<u4>(o);
+      } else {
+        const b8 o = {(__bf16)x.lo[0], (__bf16)x.lo[1], (__bf16)x.lo[2], (__bf16)x.lo[3],
+                      (__bf16)x.hi[0], (__bf16)x.hi[1], (__bf16)x.hi[2], (__bf16)x.hi[3]};
+        w = bit_cast<u4>(o);
+      }
     }
     sm_q[step * 64 + lane] = live ? w : u4{0, 0, 0, 0};
   }
@@ -187,14 +225,34 @@ __device__ __forceinline__ void pv_block(const u4 (&vreg)[D / 16], const f4 (&p)
 // reference max (exp2 domain), this lane's share of the sum (lane (n, g): head n,
 // tokens 4 g .. 4 g + 3 of every 16) and the unnormalised accumulators (channels
 // 16 * db + 4 * g .. + 3 of head n). Keys outside [vlo, p_hi) are masked.
-// stage() leaves the Q operands in sm_q; it runs once the loads of the first block are under way.
+// The caller has requested block `first` into kreg / vreg (request_first_block) and left the Q
+// operands in sm_q while those loads were under way.
 // patch_blk: a block one of whose rows is not in the cache yet (-1: none); patch(kreg, vreg) puts that
 // row into the block's registers once they are loaded.
-template <int KV, int IO, int D, class Stage, class Patch>
+template <int D>
+__device__ __forceinline__ void request_first_block(u4 (&kreg)[D / 16], u4 (&vreg)[D / 16], __amdgpu_buffer_rsrc_t krsrc,
+                                                    __amdgpu_buffer_rsrc_t vrsrc, bool streams, int first, int lane) {
+  // `first` is wave-uniform (the caller has taken it through readfirstlane) and is the very value the block
+  // loop starts from. A wave that streams nothing gets zeros, so that the registers hold defined values on
+  // every path.
+  if (streams) {
+    load_plane_block<D>(kreg, krsrc, first * (64 * D), lane * 16);
+    load_plane_block<D>(vreg, vrsrc, first * (64 * D), lane * 16);
+  } else {
+    const u4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < D / 16; ++i) kreg[i] = zero;
+#pragma unroll
+    for (int i = 0; i < D / 16; ++i) vreg[i] = zero;
+  }
+}
+
+template <int KV, int IO, int D, class Patch>
 __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buffer_rsrc_t krsrc,
-                                              __amdgpu_buffer_rsrc_t vrsrc, int first, int blk_end, int step, int vlo,
-                                              int p_hi, const u4* sm_q, int patch_blk, Stage&& stage, Patch&& patch,
-                                              int lane, float& m_run, float& l_run, f4 (&acc)[D / 16]) {
+                                              __amdgpu_buffer_rsrc_t vrsrc, u4 (&kreg)[D / 16], u4 (&vreg)[D / 16],
+                                              int first, int blk_end, int step, int vlo, int p_hi, const u4* sm_q,
+                                              int patch_blk, Patch&& patch, int lane, float& m_run, float& l_run,
+                                              f4 (&acc)[D / 16]) {
   constexpr int VB = KvT<KV>::VB, NT = VB / 16, NL = D / 16;
   constexpr int kBlockBytes = 64 * D;
   const int g = lane >> 4;
@@ -202,13 +260,7 @@ __device__ __forceinline__ void stream_blocks(const DecodeArgs& a, __amdgpu_buff
   // Rolling prefetch: the K registers are refilled with the next block as soon
   // as the QK^T product has consumed them, the V registers right after P.V, so
   // 16 to 32 KiB per wave are in flight while it computes.
-  u4 kreg[NL], vreg[NL];
-  int blk = __builtin_amdgcn_readfirstlane(first);
-  if (blk < blk_end) {
-    load_plane_block<D>(kreg, krsrc, blk * kBlockBytes, lane_off);
-    load_plane_block<D>(vreg, vrsrc, blk * kBlockBytes, lane_off);
-  }
-  stage();
+  int blk = first;  // (wave-uniform: the caller's readfirstlane)
 
   m_run = -INFINITY;
   l_run = 0.f;
@@ -447,6 +499,10 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
   float m_run, l_run;
   f4 acc[NL];
   using io_t = typename IoT<IO>::type;
+  // The first block's loads go out before anything else (a helper wave of a PRE workgroup streams nothing).
+  u4 kreg[NL], vreg[NL];
+  const int first_blk = __builtin_amdgcn_readfirstlane(p_lo / VB + wave);
+  request_first_block<D>(kreg, vreg, krsrc, vrsrc, wave < NW && first_blk < blk_end, first_blk, lane);
   if constexpr (PRE) {
     static_assert(D == kRowD, "row helpers are written for head_dim 256");
     constexpr int ESZ = KV == kF32 ? 4 : (KV == kI8 ? 1 : 2);
@@ -458,9 +514,10 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
     uint8_t* sm_vrow = sm_krow + D * ESZ;
     const int t = kv_len - 1;
     const bool owns_row = p_hi == kv_len;  // exactly one partition per sequence and KV head
-    // (always_inline: called from two places, the lambda was compiled as a function otherwise, and a sixteenth of
-    // the outputs came out wrong)
-    auto rows = [&]() __attribute__((always_inline)) {
+    // The rows: one copy of the code, at kernel scope, run by every wave of the workgroup (attention waves
+    // and helper waves alike) and closed by the workgroup's one barrier, which all NWP waves reach exactly
+    // once.
+    {
       const int nrows = G + (owns_row ? 2 : 0);  // G query rows, then the key and the value row
       constexpr int kMaxRows = (kMaxGroup + 2 + NWP - 1) / NWP;
       const int d0 = 2 * lane, d1 = D / 2 + 2 * lane;
@@ -498,20 +555,14 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
           }
         }
       }
-      __syncthreads();
-    };
-    if (wave >= NW) {  // a helper wave: its share of the rows, nothing else
-      rows();
-      return;
     }
-    auto stage = [&]() __attribute__((always_inline)) {
-      rows();
-      stage_q<KV, IO, D>(sm_q, a, sm_rows, kvh, seq, layer, lane);
-    };
+    __syncthreads();
+    if (wave >= NW) return;  // a helper wave: its share of the rows, nothing else
+    stage_q<KV, IO, D>(sm_q, a, sm_rows, kvh, seq, layer, lane);
     // Row t in the registers of its block. K: chunk c of the row is the 16 bytes of lane (t % 16, g) in load
     // (t % VB) / 16 * KPT + j with c = 4 j + g. V: element d of the row sits in lane (d % 16, (t % 16) / 4), load
     // d / 16, at element slot 4 * ((t % VB) / 16) + t % 4 of the lane's 16 bytes.
-    auto patch = [&](u4 (&kreg)[NL], u4 (&vreg)[NL]) __attribute__((always_inline)) {
+    auto patch = [&](u4 (&kr)[NL], u4 (&vr)[NL]) __attribute__((always_inline)) {
       const int tb = t % VB;
       const int tile = tb >> 4;
       const bool k_lane = (lane & 15) == (tb & 15);
@@ -521,16 +572,22 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
 #pragma unroll
           for (int j = 0; j < KPT; ++j) {
             const u4 fresh = *reinterpret_cast<const u4*>(sm_krow + (4 * j + g) * 16);
-            kreg[T * KPT + j] = k_lane ? fresh : kreg[T * KPT + j];
+            kr[T * KPT + j] = k_lane ? fresh : kr[T * KPT + j];
           }
         }
       }
       const int byte0 = (4 * tile + (tb & 3)) * ESZ;  // of the lane's 16 bytes
       const unsigned in_word = ESZ == 4 ? 0xffffffffu : ((ESZ == 2 ? 0xffffu : 0xffu) << (8 * (byte0 & 3)));
       const bool v_lane = g == ((tb & 15) >> 2);
-      unsigned mask[4];
+      // The row's element slot in the lane's 16 bytes, as whole-vector operations on purpose. Written element
+      // by element (vr[db][w] = ... for one w) this compiler's register allocator gave registers of the patched
+      // group to the softmax as temporaries before the matrix instruction that reads the group: a sixteenth of
+      // the outputs came out wrong (first seen as "wrong unless a lambda is forced inline": any change of the
+      // code's shape moved it). check_decode_kernels.py looks for that pattern in every build.
+      u4 mask;
 #pragma unroll
       for (int w = 0; w < 4; ++w) mask[w] = (v_lane && w == (byte0 >> 2)) ? in_word : 0u;
+      const u4 keep = ~mask;
 #pragma unroll
       for (int db = 0; db < NL; ++db) {
         const uint8_t* src = sm_vrow + (16 * db + n) * ESZ;
@@ -539,17 +596,17 @@ __global__ void __launch_bounds__((decode_wg_waves<NW, PRE>()) * 64, 2) decode_a
         else if constexpr (ESZ == 2) e = *reinterpret_cast<const uint16_t*>(src);
         else e = *src;
         e <<= 8 * (byte0 & 3);
-#pragma unroll
-        for (int w = 0; w < 4; ++w) vreg[db][w] = (vreg[db][w] & ~mask[w]) | (e & mask[w]);
+        const u4 ev = {e, e, e, e};
+        vr[db] = (vr[db] & keep) | (ev & mask);
       }
     };
-    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, owns_row ? t / VB : -1, stage,
+    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, kreg, vreg, first_blk, blk_end, NW, vlo, p_hi, sm_q, owns_row ? t / VB : -1,
                              patch, lane, m_run, l_run, acc);
   } else {
     const io_t* q_rows = reinterpret_cast<const io_t*>(a.q) + ((int64_t)item * a.hq + kvh * a.group) * D;
-    auto stage = [&]() __attribute__((always_inline)) { stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane); };
+    stage_q<KV, IO, D>(sm_q, a, q_rows, kvh, seq, layer, lane);
     auto patch = [](u4 (&)[NL], u4 (&)[NL]) {};
-    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, p_lo / VB + wave, blk_end, NW, vlo, p_hi, sm_q, -1, stage, patch, lane, m_run,
+    stream_blocks<KV, IO, D>(a, krsrc, vrsrc, kreg, vreg, first_blk, blk_end, NW, vlo, p_hi, sm_q, -1, patch, lane, m_run,
                              l_run, acc);
   }
   float l_tot = wave_xor_add(l_run, 16);
@@ -686,17 +743,22 @@ hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t 
 
 bool decode_supported(int kv_dtype, int io_dtype, int head_dim) {
   if (head_dim != 256) return false;
-  if (kv_dtype == kI8) return io_dtype == kF16;
-  return kv_dtype == io_dtype;
+  if (io_dtype != kF32 && io_dtype != kF16 && io_dtype != kBF16) return false;
+  if (kv_dtype == kI8) return true;                      // int8 cache: any activation type
+  return kv_dtype == io_dtype || (io_dtype == kF32 && (kv_dtype == kF16 || kv_dtype == kBF16));
 }
 
 hipError_t launch_decode(const DecodeArgs& a, int kv_dtype, int io_dtype, const DecodeTuning& tuning,
                          hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
-  switch (kv_dtype) {
-    case kF32: return launch_typed<kF32, kF32, 256>(a, tuning, stream, ev0, ev1);
-    case kF16: return launch_typed<kF16, kF16, 256>(a, tuning, stream, ev0, ev1);
-    case kBF16: return launch_typed<kBF16, kBF16, 256>(a, tuning, stream, ev0, ev1);
-    case kI8: return launch_typed<kI8, kF16, 256>(a, tuning, stream, ev0, ev1);
+  switch (kv_dtype * 4 + io_dtype) {
+    case kF32 * 4 + kF32: return launch_typed<kF32, kF32, 256>(a, tuning, stream, ev0, ev1);
+    case kF16 * 4 + kF16: return launch_typed<kF16, kF16, 256>(a, tuning, stream, ev0, ev1);
+    case kF16 * 4 + kF32: return launch_typed<kF16, kF32, 256>(a, tuning, stream, ev0, ev1);
+    case kBF16 * 4 + kBF16: return launch_typed<kBF16, kBF16, 256>(a, tuning, stream, ev0, ev1);
+    case kBF16 * 4 + kF32: return launch_typed<kBF16, kF32, 256>(a, tuning, stream, ev0, ev1);
+    case kI8 * 4 + kF16: return launch_typed<kI8, kF16, 256>(a, tuning, stream, ev0, ev1);
+    case kI8 * 4 + kBF16: return launch_typed<kI8, kBF16, 256>(a, tuning, stream, ev0, ev1);
+    case kI8 * 4 + kF32: return launch_typed<kI8, kF32, 256>(a, tuning, stream, ev0, ev1);
   }
   return hipErrorInvalidValue;
 }

@@ -70,10 +70,12 @@ __device__ __forceinline__ void cvt_i8x16_to_h8x2(u4 w, h8& lo, h8& hi) {
 }
 
 // bfloat16 bits -> the IEEE half that a V plane of a bfloat16 cache stores (exact for
-// 2^-17 <= |v| <= 65504, saturating above, nearest multiple of 2^-24 below), and back.
+// 2^-17 <= |v| <= 65504, finite values above saturate, nearest multiple of 2^-24 below), and back.
+// NaN and +-infinity pass through as NaN and +-infinity (fminf / fmaxf would turn a NaN into a bound).
 __device__ __forceinline__ uint16_t bf16_bits_to_half_bits(uint16_t b) {
   const float f = __uint_as_float((uint32_t)b << 16);
-  const _Float16 h = (_Float16)fminf(fmaxf(f, -65504.f), 65504.f);  // (NaN stays NaN)
+  const bool finite = (b & 0x7F80u) != 0x7F80u;
+  const _Float16 h = (_Float16)(finite ? fminf(fmaxf(f, -65504.f), 65504.f) : f);
   return bit_cast<uint16_t>(h);
 }
 __device__ __forceinline__ uint16_t half_bits_to_bf16_bits(uint16_t hb) {

@@ -87,6 +87,8 @@ struct mi355_attn {
   float* d_pf_acc = nullptr;   // prefill key split: parts of split tiles, allocated on first use
   float* d_pf_ml = nullptr;
   size_t pf_rows = 0;          // rows (of head_dim / of 2 floats) the two hold
+  void* d_q_stage = nullptr;   // prefill with float32 activations over a 16-bit cache: the queries in the cache's type
+  size_t q_stage_bytes = 0;
   int prefill_key_split = -1;  // < 0 by rule, 0 off, > 0 key blocks per work item
   int prefill_rows16 = -1;     // which prefill kernel: 1 the one on 16x16x32 MFMAs, 0 the one on 32x32x16, < 0 by rule
   // the step before attention: per-layer constants in HBM and what is switched on
@@ -261,10 +263,8 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
   if (new_rows) {
     if (!new_rows->k || !new_rows->v) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null k or v");
-    if (batch > kInlineItems)
-      return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
-                  "mi355_attn_decode_step takes up to %d sequences per call (got %d): call it in groups, or "
-                  "mi355_attn_pre_attention per sequence and mi355_attn_decode",
+    if (batch > kInlineItems)  // (mi355_attn_decode_step cuts larger batches into launches of this size)
+      return fail(error_msg, MI355_ATTN_INTERNAL, "a fused decode step launch holds up to %d sequences (got %d)",
                   kInlineItems, batch);
   }
   if (no_alloc && h->cfg.host_io)
@@ -435,6 +435,18 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.max_workgroups = h->prefill_workgroups;
     a.rows16 = h->prefill_rows16;
     a.host_window = h->window.data();
+    if (h->cfg.io_dtype != h->cfg.kv_dtype) {
+      const size_t need = (size_t)n_layers * n * h->cfg.num_q_heads * h->cfg.head_dim * kv_size(h);
+      if (h->q_stage_bytes < need) {
+        HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+        if (h->d_q_stage) HIP_OR_RETURN(hipFree(h->d_q_stage));
+        h->d_q_stage = nullptr;
+        h->q_stage_bytes = 0;
+        HIP_OR_RETURN(hipMalloc(&h->d_q_stage, need));
+        h->q_stage_bytes = need;
+      }
+      a.q_stage = h->d_q_stage;
+    }
     PrefillSplit split = plan_prefill_split(a, h->prefill_key_split);
     constexpr size_t kSplitRowsMax = (size_t)256 << 10;  // 256 Ki rows = 258 MiB at head_dim 256
     if (split.kchunk > 0 && split.rows > kSplitRowsMax && h->prefill_key_split < 0) split = PrefillSplit{};
@@ -525,7 +537,8 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
                 c->io_dtype);
   if (!decode_supported(c->kv_dtype, c->io_dtype, c->head_dim))
     return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
-                "kv_dtype %d with io_dtype %d (supported: equal f32/f16/bf16, or int8 cache with f16 io)",
+                "kv_dtype %d with io_dtype %d (supported: equal f32 / f16 / bf16; f16 or bf16 cache with f32 io; int8 "
+                "cache with f16, bf16 or f32 io)",
                 c->kv_dtype, c->io_dtype);
   if (c->softcap < 0.f || c->scale < 0.f)
     return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "scale and softcap must be >= 0");
@@ -650,6 +663,7 @@ void mi355_attn_destroy(mi355_attn* h) {
   free_prefill_plans(&h->pf_plans);
   if (h->d_pf_acc) (void)hipFree(h->d_pf_acc);
   if (h->d_pf_ml) (void)hipFree(h->d_pf_ml);
+  if (h->d_q_stage) (void)hipFree(h->d_q_stage);
   if (h->d_transform) (void)hipFree(h->d_transform);
   if (h->ws_acc) (void)hipFree(h->ws_acc);
   if (h->ws_ml) (void)hipFree(h->ws_ml);
@@ -866,8 +880,46 @@ int mi355_attn_prefill_plan_probe(int32_t n_layers, int32_t n, int32_t q_pos0, i
 int mi355_attn_decode_step(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens, int32_t batch,
                            const void* q, const void* k, const void* v, void* out, int32_t num_splits,
                            char** error_msg) {
-  const NewRows rows{k, v};
-  return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg, /*no_alloc=*/false, &rows);
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (batch <= kInlineItems) {
+    const NewRows rows{k, v};
+    return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg, /*no_alloc=*/false, &rows);
+  }
+  // More sequences than one launch carries in its argument block: launches of kInlineItems sequences each, queued
+  // back to back. Everything that can be refused is checked for the whole batch first, so that a call either
+  // runs all of its launches or none.
+  if (int rc = check_layers(h, layer, 1, error_msg)) return rc;
+  if (!kv_lens || !q || !k || !v || !out) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null kv_lens, q, k, v or out");
+  if (batch > h->cfg.max_seqs)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "batch %d outside [1, max_seqs=%d]", batch, h->cfg.max_seqs);
+  if (num_splits < 0 || num_splits > kMaxSplits)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "num_splits %d outside [0, %d]", num_splits, kMaxSplits);
+  std::vector<int32_t> ids(batch);
+  std::vector<char> named(h->cfg.max_seqs, 0);
+  for (int b = 0; b < batch; ++b) {
+    const int seq = seq_ids ? seq_ids[b] : b;
+    if (seq < 0 || seq >= h->cfg.max_seqs)
+      return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq_ids[%d]=%d outside [0, %d)", b, seq, h->cfg.max_seqs);
+    if (named[seq]) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "seq_ids names sequence %d twice (entry %d)", seq, b);
+    named[seq] = 1;
+    ids[b] = seq;
+    const int len = kv_lens[b];
+    if (len < 1 || len > h->cfg.max_tokens)
+      return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "kv_lens[%d]=%d outside [1, max_tokens=%d]", b, len, h->cfg.max_tokens);
+    if (len - 1 > h->filled[(size_t)layer * h->cfg.max_seqs + seq])
+      return fail(error_msg, MI355_ATTN_OUT_OF_RANGE, "kv_lens[%d]=%d but only %d rows of layer %d, sequence %d were appended",
+                  b, len, h->filled[(size_t)layer * h->cfg.max_seqs + seq], layer, seq);
+  }
+  const size_t q_row = (size_t)h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
+  const size_t kv_row = (size_t)h->cfg.num_kv_heads * h->cfg.head_dim * io_size(h);
+  for (int b0 = 0; b0 < batch; b0 += kInlineItems) {
+    const int nb = std::min<int>(kInlineItems, batch - b0);
+    const NewRows rows{static_cast<const uint8_t*>(k) + b0 * kv_row, static_cast<const uint8_t*>(v) + b0 * kv_row};
+    if (int rc = decode_impl(h, layer, 1, ids.data() + b0, kv_lens + b0, nb, static_cast<const uint8_t*>(q) + b0 * q_row,
+                             static_cast<uint8_t*>(out) + b0 * q_row, num_splits, error_msg, /*no_alloc=*/false, &rows))
+      return rc;
+  }
+  return MI355_ATTN_OK;
 }
 
 int mi355_attn_decode_noalloc(mi355_attn* h, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,

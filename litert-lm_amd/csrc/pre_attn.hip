@@ -87,12 +87,15 @@ hipError_t launch_pre_attention(const PreAttentionArgs& a, int kv_dtype, int io_
                                 hipEvent_t ev0, hipEvent_t ev1) {
   if (a.n <= 0) return hipSuccess;
   if (a.geom.head_dim != kD) return hipErrorInvalidValue;
-  if (kv_dtype == kI8 && io_dtype == kF16) return launch_typed<kF16, kI8>(a, stream, ev0, ev1);
-  if (kv_dtype != io_dtype) return hipErrorInvalidValue;
-  switch (io_dtype) {
-    case kF32: return launch_typed<kF32, kF32>(a, stream, ev0, ev1);
-    case kF16: return launch_typed<kF16, kF16>(a, stream, ev0, ev1);
-    case kBF16: return launch_typed<kBF16, kBF16>(a, stream, ev0, ev1);
+  switch (kv_dtype * 4 + io_dtype) {
+    case kF32 * 4 + kF32: return launch_typed<kF32, kF32>(a, stream, ev0, ev1);
+    case kF16 * 4 + kF16: return launch_typed<kF16, kF16>(a, stream, ev0, ev1);
+    case kF16 * 4 + kF32: return launch_typed<kF32, kF16>(a, stream, ev0, ev1);
+    case kBF16 * 4 + kBF16: return launch_typed<kBF16, kBF16>(a, stream, ev0, ev1);
+    case kBF16 * 4 + kF32: return launch_typed<kF32, kBF16>(a, stream, ev0, ev1);
+    case kI8 * 4 + kF16: return launch_typed<kF16, kI8>(a, stream, ev0, ev1);
+    case kI8 * 4 + kBF16: return launch_typed<kBF16, kI8>(a, stream, ev0, ev1);
+    case kI8 * 4 + kF32: return launch_typed<kF32, kI8>(a, stream, ev0, ev1);
     default: return hipErrorInvalidValue;
   }
 }

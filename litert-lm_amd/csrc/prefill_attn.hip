@@ -66,6 +66,17 @@ struct El<kBF16> {
   static __device__ __forceinline__ f16v mfma(vec8 a, vec8 b, f16v c) { return mfma32_bf16(a, b, c); }
 };
 
+// Output element type: the cache's own 16-bit type, or float32 for float32 activations (the queries of such a
+// call are rounded to the cache's type by convert_queries_kernel before the attention kernel runs).
+template <int OUT>
+struct OutEl;
+template <>
+struct OutEl<kF32> { using type = float; };
+template <>
+struct OutEl<kF16> { using type = _Float16; };
+template <>
+struct OutEl<kBF16> { using type = __bf16; };
+
 // Key (0..31, within a block) that MFMA row m of S^T stands for.
 __device__ __forceinline__ int key_of_row(int m) { return 16 * ((m >> 3) & 1) + 8 * (m >> 4) + (m & 7); }
 
@@ -108,7 +119,7 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-template <int DT, int D, int HPB, bool CAP>
+template <int DT, int OUT, int D, int HPB, bool CAP>
 __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
@@ -564,6 +575,32 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
         *reinterpret_cast<u4*>(a.ws_acc + slot * D + lane * 4) = w;
       }
     }
+  } else if constexpr (OUT == kF32) {
+    // float32 rows: the same route as the parts of a split tile, normalised, to the output
+    constexpr int kRowStrideF = 4 * D + 16;
+    uint8_t* const patch = smem + wave * (kStretch * kRowStrideF) + (wave >= 2 ? 16384 : 0);
+    const float l_tot = wave_xor_add(l_run0, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+    for (int dp = 0; dp < NDP; ++dp) {
+#pragma unroll
+      for (int aa = 0; aa < 4; ++aa) {
+        f4 o;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) o[b] = acc0[dp][4 * aa + b] * inv;
+        *reinterpret_cast<f4*>(patch + n * kRowStrideF + (32 * dp + 8 * aa + 4 * hh) * 4) = o;
+      }
+    }
+    const int row_base = my_pos0 - a.q_pos0;
+#pragma unroll 4
+    for (int r = 0; r < kStretch; ++r) {
+      const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStrideF + lane * 16);
+      const int row = row_base + r;
+      if (row < a.n) {
+        float* orow = reinterpret_cast<float*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
+        *reinterpret_cast<u4*>(orow + lane * 4) = w;
+      }
+    }
   } else {
     constexpr int kRowStride = 2 * D + 16;
     uint8_t* const patch = smem + wave * (kStretch * kRowStride);
@@ -638,8 +675,7 @@ constexpr int kOpAheadV = 4;
 template <int D>
 constexpr int prefill16_lds_bytes() { return (kKStages16 + kVStages16) * 64 * D; }  // 80 KiB: two workgroups fill a CU's LDS
 
-template <int DT, int D, int HPB, bool CAP>
-
+template <int DT, int OUT, int D, int HPB, bool CAP>
 __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
@@ -956,9 +992,9 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
       float l_tot = wave_xor_add(l_run[u], 16);
       l_tot = wave_xor_add(l_tot, 32);
       const int row = my_pos0 + kRows16 * u + n - a.q_pos0;
-      // (lane n = 0 has a row to store: the wave issues the sub-tile's store instructions, NL / 2 of 16 bytes, or
-      // NL + 1 for a part of a split tile)
-      if (wave_pos0 + kRows16 * u - a.q_pos0 < a.n) stores_after_q += it.split ? NL : NL / 2;
+      // (lane n = 0 has a row to store: the wave issues the sub-tile's store instructions, NL / 2 of 16 bytes, NL
+      // for float32 output, or NL + 1 for a part of a split tile)
+      if (wave_pos0 + kRows16 * u - a.q_pos0 < a.n) stores_after_q += (it.split || OUT == kF32) ? NL : NL / 2;
       if (row < a.n) {
         if (it.split) {
           const int64_t slot = (((int64_t)it.li * a.n + row) * a.hq + it.head) * smax + it.part;
@@ -969,30 +1005,41 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
         }
       }
       if (!it.split) {
-        // Pairs of channel tiles trade halves between the lanes g and g ^ 1 of a query (v_permlane16_swap), so
-        // that a lane ends up with 8 consecutive channels, 16 bytes, and the four lanes of a query with 64
-        // consecutive bytes per store instruction (8-byte pieces straight from the MFMA layout cost four
-        // times the write requests). Every lane takes part in the trade; only rows that exist are stored.
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        uint32_t packed[NL][2];
+        if constexpr (OUT == kF32) {
+          // float32 output: a lane's four channels of a tile are 16 bytes already, the four lanes of a query
+          // 64 consecutive bytes per store instruction
+          float* orow = reinterpret_cast<float*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + 4 * g;
 #pragma unroll
-        for (int db = 0; db < NL; ++db) {
-          elem_t o[4];
+          for (int db = 0; db < NL; ++db) {
+            const f4 o = acc[u][db] * inv;
+            if (row < a.n) *reinterpret_cast<f4*>(orow + 16 * db) = o;
+          }
+        } else {
+          // Pairs of channel tiles trade halves between the lanes g and g ^ 1 of a query (v_permlane16_swap), so
+          // that a lane ends up with 8 consecutive channels, 16 bytes, and the four lanes of a query with 64
+          // consecutive bytes per store instruction (8-byte pieces straight from the MFMA layout cost four
+          // times the write requests). Every lane takes part in the trade; only rows that exist are stored.
+          uint32_t packed[NL][2];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (elem_t)(acc[u][db][e] * inv);
-          const u2 w = *reinterpret_cast<const u2*>(o);
-          packed[db][0] = w[0];
-          packed[db][1] = w[1];
-        }
-        // lanes g = 0, 2 keep tile 2k (channels 32k + 4g .. + 7), lanes g = 1, 3 tile 2k + 1 (32k + 16 + 4(g - 1) .. + 7)
-        const int first = (g & 1) * 16 + (g >> 1) * 8;
-        elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + first;
+          for (int db = 0; db < NL; ++db) {
+            elem_t o[4];
 #pragma unroll
-        for (int k = 0; k < NL / 2; ++k) {
-          const auto lo = __builtin_amdgcn_permlane16_swap(packed[2 * k][0], packed[2 * k + 1][0], false, false);
-          const auto hi = __builtin_amdgcn_permlane16_swap(packed[2 * k][1], packed[2 * k + 1][1], false, false);
-          const u4 w = {lo[0], hi[0], lo[1], hi[1]};
-          if (row < a.n) *reinterpret_cast<u4*>(orow + 32 * k) = w;
+            for (int e = 0; e < 4; ++e) o[e] = (elem_t)(acc[u][db][e] * inv);
+            const u2 w = *reinterpret_cast<const u2*>(o);
+            packed[db][0] = w[0];
+            packed[db][1] = w[1];
+          }
+          // lanes g = 0, 2 keep tile 2k (channels 32k + 4g .. + 7), lanes g = 1, 3 tile 2k + 1 (32k + 16 + 4(g - 1) .. + 7)
+          const int first = (g & 1) * 16 + (g >> 1) * 8;
+          elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + first;
+#pragma unroll
+          for (int k = 0; k < NL / 2; ++k) {
+            const auto lo = __builtin_amdgcn_permlane16_swap(packed[2 * k][0], packed[2 * k + 1][0], false, false);
+            const auto hi = __builtin_amdgcn_permlane16_swap(packed[2 * k][1], packed[2 * k + 1][1], false, false);
+            const u4 w = {lo[0], hi[0], lo[1], hi[1]};
+            if (row < a.n) *reinterpret_cast<u4*>(orow + 32 * k) = w;
+          }
         }
       }
     }
@@ -1010,9 +1057,9 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
 // Combines the parts of split tiles: grid (query head, row, layer), one thread
 // per channel. Rows of tiles that were not split have been written by the
 // attention kernel itself.
-template <int DT, int D>
+template <int OUT, int D>
 __global__ void __launch_bounds__(D) prefill_merge_kernel(const PrefillArgs a, int rows_per_tile) {
-  using elem_t = typename El<DT>::type;
+  using elem_t = typename OutEl<OUT>::type;
   const int head = blockIdx.x, row = blockIdx.y, li = blockIdx.z, d = threadIdx.x;
   const int window = a.layer_window[a.layer_begin + li];
   const int wg_pos0 = a.q_pos0 + (row / rows_per_tile) * rows_per_tile;
@@ -1035,46 +1082,61 @@ __global__ void __launch_bounds__(D) prefill_merge_kernel(const PrefillArgs a, i
   reinterpret_cast<elem_t*>(a.out)[(((int64_t)li * a.n + row) * a.hq + head) * D + d] = (elem_t)(L > 0.f ? A / L : 0.f);
 }
 
-template <int DT, int D, int HPB, bool CAP>
+// float32 queries rounded (to nearest even) to the element type of the cache, 8 per thread: what the
+// matrix cores take. One pass over the call's query rows in front of the attention kernel.
+template <int DT>
+__global__ void __launch_bounds__(256) convert_queries_kernel(const float* __restrict__ src, void* __restrict__ dst, int64_t n8) {
+  using vec8 = typename El<DT>::vec8;
+  using elem_t = typename El<DT>::type;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n8) return;
+  const f4 x0 = *reinterpret_cast<const f4*>(src + 8 * i), x1 = *reinterpret_cast<const f4*>(src + 8 * i + 4);
+  vec8 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { o[e] = (elem_t)x0[e]; o[4 + e] = (elem_t)x1[e]; }
+  reinterpret_cast<vec8*>(dst)[i] = o;
+}
+
+template <int DT, int OUT, int D, int HPB, bool CAP>
 hipError_t launch_variant(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill_lds_bytes<D>();
   // more than 64 KiB of LDS has to be requested once per kernel (callers on several threads may both
   // make the request; it is idempotent)
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, D, HPB, CAP>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn_kernel<DT, OUT, D, HPB, CAP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
     configured.store(true, std::memory_order_release);
   }
   // ev0/ev1 ride on the dispatch: the kernel's own begin / end timestamps
-  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, D, HPB, CAP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
+  hipExtLaunchKernelGGL((prefill_attn_kernel<DT, OUT, D, HPB, CAP>), grid, dim3(kWaves * 64), kLds, stream, ev0, ev1, 0,
                         a);
   return hipGetLastError();
 }
 
-template <int DT, int D, int HPB, bool CAP>
+template <int DT, int OUT, int D, int HPB, bool CAP>
 hipError_t launch_variant16(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   constexpr int kLds = prefill16_lds_bytes<D>();
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn16_kernel<DT, D, HPB, CAP>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attn16_kernel<DT, OUT, D, HPB, CAP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return e;
     configured.store(true, std::memory_order_release);
   }
-  hipExtLaunchKernelGGL((prefill_attn16_kernel<DT, D, HPB, CAP>), grid, dim3(kWaves16 * 64), kLds, stream, ev0,
+  hipExtLaunchKernelGGL((prefill_attn16_kernel<DT, OUT, D, HPB, CAP>), grid, dim3(kWaves16 * 64), kLds, stream, ev0,
                         ev1, 0, a);
   return hipGetLastError();
 }
 
-template <int DT, int D, int HPB>
+template <int DT, int OUT, int D, int HPB>
 hipError_t launch_hpb(const PrefillArgs& a, dim3 grid, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   if (a.rows16)
-    return a.softcap > 0.f ? launch_variant16<DT, D, HPB, true>(a, grid, stream, ev0, ev1)
-                           : launch_variant16<DT, D, HPB, false>(a, grid, stream, ev0, ev1);
-  return a.softcap > 0.f ? launch_variant<DT, D, HPB, true>(a, grid, stream, ev0, ev1)
-                         : launch_variant<DT, D, HPB, false>(a, grid, stream, ev0, ev1);
+    return a.softcap > 0.f ? launch_variant16<DT, OUT, D, HPB, true>(a, grid, stream, ev0, ev1)
+                           : launch_variant16<DT, OUT, D, HPB, false>(a, grid, stream, ev0, ev1);
+  return a.softcap > 0.f ? launch_variant<DT, OUT, D, HPB, true>(a, grid, stream, ev0, ev1)
+                         : launch_variant<DT, OUT, D, HPB, false>(a, grid, stream, ev0, ev1);
 }
 
 // Key blocks of tile `t` of a layer with window `w` (0: global): the kernels' own arithmetic.
@@ -1325,7 +1387,7 @@ hipError_t plan_for(const PrefillArgs& a, int hpb, int wgs, int cus, PrefillPlan
   return hipSuccess;
 }
 
-template <int DT, int D>
+template <int DT, int OUT, int D>
 hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
   const int G = a.group;
   const int hpb = (G % 4 == 0) ? 4 : ((G % 2 == 0) ? 2 : 1);
@@ -1342,6 +1404,16 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
   }
   PrefillArgs b = a;
   b.use_order = 0;
+  if constexpr (OUT != DT) {
+    // float32 activations: the queries go through the staging rows in the cache's type first
+    if (!a.q_stage) return hipErrorInvalidValue;
+    const int64_t n8 = (int64_t)a.n_layers * a.n * a.hq * D / 8;
+    hipLaunchKernelGGL((convert_queries_kernel<DT>), dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const float*>(a.q), a.q_stage, n8);
+    hipError_t ce = hipGetLastError();
+    if (ce != hipSuccess) return ce;
+    b.q = a.q_stage;
+  }
 
   const int units = a.n_layers * a.geom.hkv * (G / hpb);
   if (units <= kPrefillOrderUnits && a.host_window) {
@@ -1399,9 +1471,9 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
     if (pe != hipSuccess) return pe;
     b.plan = plans->d_words[plan_slot];
   }
-  hipError_t err = hpb == 4   ? launch_hpb<DT, D, 4>(b, grid, stream, ev0, ev1)
-                   : hpb == 2 ? launch_hpb<DT, D, 2>(b, grid, stream, ev0, ev1)
-                              : launch_hpb<DT, D, 1>(b, grid, stream, ev0, ev1);
+  hipError_t err = hpb == 4   ? launch_hpb<DT, OUT, D, 4>(b, grid, stream, ev0, ev1)
+                   : hpb == 2 ? launch_hpb<DT, OUT, D, 2>(b, grid, stream, ev0, ev1)
+                              : launch_hpb<DT, OUT, D, 1>(b, grid, stream, ev0, ev1);
   if (err == hipSuccess && plan_slot >= 0) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     err = hipStreamIsCapturing(stream, &capturing);
@@ -1410,7 +1482,7 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
     else if (err == hipSuccess) plans->pinned[plan_slot] = true;
   }
   if (err != hipSuccess || a.kchunk <= 0) return err;
-  hipLaunchKernelGGL((prefill_merge_kernel<DT, D>), dim3(a.hq, a.n, a.n_layers), dim3(D), 0, stream, b, kStretch * pt);
+  hipLaunchKernelGGL((prefill_merge_kernel<OUT, D>), dim3(a.hq, a.n, a.n_layers), dim3(D), 0, stream, b, kStretch * pt);
   return hipGetLastError();
 }
 
@@ -1513,14 +1585,15 @@ PrefillSplit plan_prefill_split(const PrefillArgs& a, int option) {
 }
 
 bool prefill_supported(int kv_dtype, int io_dtype, int head_dim) {
-  return head_dim == 256 && kv_dtype == io_dtype && (kv_dtype == kF16 || kv_dtype == kBF16);
+  return head_dim == 256 && (kv_dtype == kF16 || kv_dtype == kBF16) && (io_dtype == kv_dtype || io_dtype == kF32);
 }
 
 hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, PrefillPlans* plans, hipStream_t stream,
                           hipEvent_t ev0, hipEvent_t ev1) {
-  (void)io_dtype;
-  if (kv_dtype == kF16) return launch_typed<kF16, 256>(a, plans, stream, ev0, ev1);
-  if (kv_dtype == kBF16) return launch_typed<kBF16, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kF16 && io_dtype == kF16) return launch_typed<kF16, kF16, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kF16 && io_dtype == kF32) return launch_typed<kF16, kF32, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kBF16 && io_dtype == kBF16) return launch_typed<kBF16, kBF16, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kBF16 && io_dtype == kF32) return launch_typed<kBF16, kF32, 256>(a, plans, stream, ev0, ev1);
   return hipErrorInvalidValue;
 }
 

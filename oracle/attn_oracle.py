@@ -374,3 +374,28 @@ def rel_err_beyond_bf16_rounding(a, b) -> float:
     excess = np.maximum(np.abs(a - b) - half_ulp_bf16(b), 0.0)
     den = np.abs(b).max()
     return float(excess.max() / (den if den > 0 else 1.0))
+
+
+def bf16_bits(x) -> np.ndarray:
+    """Bit patterns (uint16) of x rounded to the nearest bfloat16, ties to even."""
+    f = np.ascontiguousarray(np.asarray(x, dtype=np.float32))
+    u = f.view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def bf16_ulp_distance(a, b) -> np.ndarray:
+    """Distance between two arrays of bfloat16 values counted in representable bfloat16 numbers
+    (0: the same number; 1: neighbours; +0 and -0 count as one number). Inputs are rounded to
+    bfloat16 first, so values that already are bfloat16 numbers pass through unchanged."""
+    def ordered(bits):
+        bits = bits.astype(np.int64)
+        return np.where(bits & 0x8000, -(bits & 0x7FFF), bits & 0x7FFF)
+    return np.abs(ordered(bf16_bits(a)) - ordered(bf16_bits(b)))
+
+
+def bf16_output_match(got, ref):
+    """How a bfloat16 result compares with the correctly rounded one, with no allowance: the share of
+    elements equal to round_bf16(ref), and the largest distance of the others in bfloat16 steps."""
+    d = bf16_ulp_distance(got, round_bf16(ref))
+    return float((d == 0).mean()), int(d.max()) if d.size else 0
+

@@ -138,6 +138,13 @@ def test_full_batch_of_64():
     drive_both(A.F16, 4, 1, lens, 2, [0], 0, 0, seed=5)
 
 
+def test_more_sequences_than_one_launch_holds():
+    say("decode_step: 150 sequences (three launches behind one call), permuted cache slots")
+    g = np.random.default_rng(9)
+    lens = [int(x) for x in g.integers(1, 120, size=150)]
+    drive_both(A.F16, 8, 2, lens, 2, [0, 40], 0, 0, seq_ids=[int(x) for x in g.permutation(150)], seed=9)
+
+
 @pytest.mark.parametrize("kv", [A.F16, A.BF16, A.I8])
 def test_long_context(kv):
     say(f"decode_step kv {kv}: context 4090 -> 4096, positions where the angles are thousands of radians")
@@ -243,9 +250,14 @@ def test_argument_checks_and_row_accounting():
         with pytest.raises(A.AttnError) as e:
             at.decode_step(0, [1, 1], q[:2], kv[:2], kv[:2], out[:2], seq_ids=[3, 3])
         assert e.value.code == A.INVALID_ARGUMENT
+        with pytest.raises(A.AttnError) as e:  # a batch cut into two launches is checked as a whole before the first
+            at.decode_step(0, [1] * 64 + [2], q[:65], kv[:65], kv[:65], out[:65])
+        assert e.value.code == A.OUT_OF_RANGE
         with pytest.raises(A.AttnError) as e:
-            at.decode_step(0, [1] * 65, q[:65], kv[:65], kv[:65], out[:65])
-        assert e.value.code == A.UNIMPLEMENTED
+            at.decode_step(0, [1] * 65, q[:65], kv[:65], kv[:65], out[:65], seq_ids=list(range(64)) + [5])
+        assert e.value.code == A.INVALID_ARGUMENT
+        at.decode_step(0, [1] * 64, q[:64], kv[:64], kv[:64], out[:64])  # (nothing of the refused calls was written)
+        at.reset()
         with pytest.raises(A.AttnError) as e:
             at.decode_step(1, [1], q[:1], kv[:1], kv[:1], out[:1])
         assert e.value.code == A.INVALID_ARGUMENT

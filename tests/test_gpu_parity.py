@@ -432,6 +432,34 @@ def test_bf16_value_planes_hold_half_precision_values():
         assert np.array_equal(got[exact], vr[exact]) and int((~exact).sum()) >= 5
 
 
+def test_bf16_value_planes_pass_non_finite_values_through():
+    """NaN and +-infinity in a V row of a bfloat16 cache come back as NaN and +-infinity (finite values beyond
+    65504 saturate; a non-finite one must not turn into a bound silently)."""
+    hkv, n = 1, 16
+    vals = np.random.default_rng(6).standard_normal((n, hkv, D)).astype(np.float32)
+    vals[3, 0, :4] = [np.inf, -np.inf, np.nan, 7.0e4]
+    with make(1, 4, hkv, n, 1, A.BF16) as at:
+        vd = torch.from_numpy(vals).to(DEV).bfloat16()
+        at.kv_append(0, 0, 0, vd, vd)
+        ko, vo = torch.zeros_like(vd), torch.zeros_like(vd)
+        at.kv_read(0, 0, 0, n, ko, vo)
+        torch.cuda.synchronize()
+        assert torch.equal(ko.view(torch.int16), vd.view(torch.int16))  # keys: bit for bit, NaN included
+        got = vo.float().cpu().numpy()
+        assert got[3, 0, 0] == np.inf and got[3, 0, 1] == -np.inf and np.isnan(got[3, 0, 2])
+        assert got[3, 0, 3] == np.float32(torch.tensor(65504.0).bfloat16().float())  # finite: saturates (read back as bf16)
+        rest = np.ones_like(vals, dtype=bool)
+        rest[3, 0, :4] = False
+        assert np.array_equal(got[rest], vd.float().cpu().numpy()[rest])
+        # the same row through the step before attention (a layer without constants: a plain append)
+        qd = torch.zeros((n, 4, D), dtype=torch.bfloat16, device=DEV)
+        at.pre_attention(0, 0, 0, qd, vd, vd, torch.empty_like(qd))
+        at.kv_read(0, 0, 0, n, ko, vo)
+        torch.cuda.synchronize()
+        got2 = vo.float().cpu().numpy()
+        assert got2[3, 0, 0] == np.inf and got2[3, 0, 1] == -np.inf and np.isnan(got2[3, 0, 2])
+
+
 @ROWS16
 def test_prefill_c2_full_size_local_and_global(rows16):
     # config 2: 1024-token chunk, Hq4/Hkv1, bf16; one local (W=512) and one global layer
