@@ -12,7 +12,8 @@ come from HBM, not from L2 / Infinity Cache.
 Prints ONE JSON line. `value` is algorithmic bytes per step / wall time per
 step with all inputs resident in HBM. Every leg is timed over a region of at
 least 50 ms whatever --steps says (`timed_steps` says how many steps that
-took). `roofline` prices the decode attention kernel alone (begin / end stamps
+took). `sustained` repeats the headline step (and, under `prefill`, the config-2
+launch) back to back for 2 s. `roofline` prices the decode attention kernel alone (begin / end stamps
 attached to each dispatch, on the stream it runs on) against the 8 TB/s HBM
 peak. `decode_graph` replays the same work from HIP graphs: the one multi-layer
 launch, and the 30 layers as 30 launches in dependency order (what a forward
@@ -39,6 +40,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 D = 256
 METRIC = "decode-attn HBM GB/s (% of 8 TB/s) + prefill-attn TFLOP/s, Gemma3n-E2B shape"
 MIN_TIMED_REGION_S = 0.05
+SUSTAINED_S = 2.0  # the headline step and the config-2 prefill launch are also run back to back for this long
 
 
 def log(*a):
@@ -129,6 +131,9 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
 
         sec, timed = time_steps(torch, step, steps, warmup)
         kms, burst_ms = kernel_ms(torch, at, step, 0)
+        # the same steps back to back for SUSTAINED_S seconds: the rate at the clocks and the memory state the part
+        # settles into under this load (the 50 ms regions above end before it does)
+        sec_long, timed_long = time_steps(torch, step, steps, 0, min_region_s=SUSTAINED_S)
         # algorithmic bytes: K and V once, Q and O once (no partials, no padding)
         per_layer = ctx * hkv * D * 2 * 2 + 2 * hq * D * 2
         step_bytes = per_layer * layers
@@ -190,6 +195,7 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
         torch.cuda.synchronize()
         at.close()
     return {"sec_per_step": sec, "timed_steps": timed, "kernel_ms": kms, "burst_ms_per_step": burst_ms,
+            "sustained_sec_per_step": sec_long, "sustained_steps": timed_long,
             "step_bytes": step_bytes, "layers": layers, "single_layer_latency_us": lat * 1e6,
             "tokens_per_s": 1.0 / sec, "graph": graph}
 
@@ -258,7 +264,7 @@ def prefill_flops(n, hq, window):
     return 4 * hq * D * pairs
 
 
-def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_layer=False, rows16=-1):
+def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_layer=False, rows16=-1, sustained=False):
     hq, hkv = 4, 1
     windows = [0 if (l + 1) % 6 == 0 else 512 for l in range(layers)]
     stream = torch.cuda.current_stream().cuda_stream
@@ -275,6 +281,7 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_
     sec, timed = time_steps(torch, step, steps, warmup)
     kms, burst_ms = kernel_ms(torch, at, step, 0)
     flops = sum(prefill_flops(n, hq, w) for w in windows)
+    sec_long, timed_long = time_steps(torch, step, steps, 0, min_region_s=SUSTAINED_S) if sustained else (float("nan"), 0)
 
     def step1(i):
         at.prefill(5, 0, 0, n, q[5], out[5])  # one global layer
@@ -293,7 +300,7 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_
     return {"workload": f"C2: 26 layers x 1024 tokens, Hq4/Hkv1, {'fp16' if half else 'bf16'}, "
                         "22 local(W=512)+4 global, one launch",
             "ms_per_step": sec * 1e3, "timed_steps": timed, "kernel_ms": kms, "burst_ms_per_step": burst_ms,
-            "flops": flops, "TFLOPs": flops / sec / 1e12,
+            "flops": flops, "TFLOPs": flops / sec / 1e12, "sustained_sec_per_step": sec_long, "sustained_steps": timed_long,
             "kernel_TFLOPs": flops / (kms * 1e-3) / 1e12,
             "frac_of_mfma_peak": flops / (kms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
             "tokens_per_s": n / sec, "single_global_layer_ms": lat1 * 1e3,
@@ -522,6 +529,12 @@ def main():
             "timing": f"every leg is timed over at least {MIN_TIMED_REGION_S} s of back-to-back steps (timed_steps >= --steps)",
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "value_is": f"algorithmic bytes per step / wall time per step over the {MIN_TIMED_REGION_S} s region (ms_per_step x "
+                    "timed_steps); `sustained` is the same step queued back to back for 2 s",
+        "sustained": {"seconds": round(dec["sustained_sec_per_step"] * dec["sustained_steps"], 3),
+                      "steps": dec["sustained_steps"], "ms_per_step": round(dec["sustained_sec_per_step"] * 1e3, 5),
+                      "GBps": round(dec["step_bytes"] / dec["sustained_sec_per_step"] / 1e9, 1),
+                      "frac_of_hbm_peak": round(dec["step_bytes"] / dec["sustained_sec_per_step"] / 1e9 / HBM_PEAK_GBS, 4)},
         "decode_steps_per_s": round(dec["tokens_per_s"], 1),
         "single_layer_latency_us": round(dec["single_layer_latency_us"], 2),
         "roofline": {
@@ -541,13 +554,17 @@ def main():
 
     if not args.no_extras:
         few, fw = max(20, args.steps // 4), max(5, args.warmup // 4)
-        pre = bench_prefill_c2(A, torch, few, fw, by_layer=not args.no_pipeline)
+        pre = bench_prefill_c2(A, torch, few, fw, by_layer=not args.no_pipeline, sustained=True)
         log(f"[bench] prefill C2: {pre['ms_per_step']:.4f} ms/step over {pre['timed_steps']} steps, "
             f"{pre['kernel_TFLOPs']:.1f} TFLOP/s kernel")
         result["prefill"] = {
             "workload": pre["workload"], "value": round(pre["TFLOPs"], 2), "unit": "TFLOP/s", "dtype": "bf16",
             "ms_per_step": round(pre["ms_per_step"], 4), "timed_steps": pre["timed_steps"],
             "prefill_tokens_per_s": round(pre["tokens_per_s"], 1),
+            "sustained": {"seconds": round(pre["sustained_sec_per_step"] * pre["sustained_steps"], 3),
+                          "steps": pre["sustained_steps"], "ms_per_step": round(pre["sustained_sec_per_step"] * 1e3, 5),
+                          "TFLOPs": round(pre["flops"] / pre["sustained_sec_per_step"] / 1e12, 2),
+                          "frac_of_mfma_peak": round(pre["flops"] / pre["sustained_sec_per_step"] / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
             "single_global_layer_ms": round(pre["single_global_layer_ms"], 4),
             "layer_by_layer": None if args.no_pipeline else {
                 "what": "the same 26 layers as 26 launches in turn (how an executor calls it); key ranges of a "

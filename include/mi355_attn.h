@@ -258,8 +258,17 @@ int mi355_attn_decode_step(mi355_attn* handle, int32_t layer, const int32_t* seq
  * kFailedPrecondition); batch x num_q_heads x num_splits <= 8192 partial results
  * (an explicit num_splits beyond that is kResourceExhausted; with num_splits = 0
  * the library chooses within the limit). All calls on one GPU share the
- * workspace: calls that overlap in time on one GPU (two handles on two streams)
- * race; calls queued on one stream do not.
+ * workspace. Calls queued on one stream never overlap. Eager calls on different
+ * streams are ordered by the library (each waits, on its stream, for the event
+ * the previous one left), so they do not overlap either. Calls recorded into HIP
+ * graphs are not ordered against anything outside their graph: replays of two
+ * graphs (or a replay and an eager call) that run at the same time on one GPU
+ * race in the workspace - keep them on one stream.
+ * Under capture (this entry point, mi355_attn_decode and mi355_attn_decode_step
+ * alike): up to 64 sequences per call (more need an upload that a capture cannot
+ * hold: kFailedPrecondition); kv_lens and seq_ids are baked into the recorded
+ * launch, so a replay attends exactly the rows of the captured call - one graph
+ * per position - and does not advance the handle's count of appended rows.
  */
 int mi355_attn_decode_noalloc(mi355_attn* handle, int32_t layer, const int32_t* seq_ids, const int32_t* kv_lens,
                               int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg);

@@ -36,7 +36,10 @@ PrefillSplit plan_prefill_split(const PrefillArgs& args, int option);
 // in which order, computed on the host (longest processing time first over the workgroups: an item's time is
 // known from its number of key blocks) and cached by launch shape. A slot's device copy is rewritten only
 // after the last launch that reads it has finished (`used`); a slot whose launch was captured into a HIP graph
-// is kept for good (`pinned`: the graph may be replayed at any time).
+// is kept for good (`pinned`: the graph may be replayed at any time). A new shape takes the least recently used
+// slot that is not pinned. A launch that cannot get a plan - a shape seen for the first time while its stream is
+// being captured, or all slots pinned - runs on the other prefill kernel, which needs none: same results to the
+// tolerance, not bit for bit.
 struct PrefillPlans {
   static constexpr int kSlots = 4;
   int32_t* d_words[kSlots] = {};
@@ -46,7 +49,8 @@ struct PrefillPlans {
   int64_t key[kSlots][8] = {};
   bool valid[kSlots] = {};
   bool pinned[kSlots] = {};
-  int next = 0;
+  uint64_t last_use[kSlots] = {};
+  uint64_t clock = 0;
 };
 void free_prefill_plans(PrefillPlans* plans);
 

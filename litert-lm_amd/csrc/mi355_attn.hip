@@ -34,6 +34,13 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 float* g_scratch_ptr[kMaxDevices] = {};  // [device]: address of `scratch` on that GPU, set once by create
+// Calls on different streams of one GPU share that GPU's `scratch`: each call waits (on its stream, not on the
+// host) for the event that the previous call left behind when that call ran on another stream, so eager calls
+// never overlap in the workspace. The events are made once per GPU by create. (Captured calls skip this: an
+// event recorded inside a capture belongs to the graph.)
+hipEvent_t g_scratch_done[kMaxDevices] = {};
+hipStream_t g_scratch_stream[kMaxDevices] = {};
+bool g_scratch_used[kMaxDevices] = {};
 
 constexpr int kRingSlots = 64;
 constexpr int kMaxSplits = kMaxDecodeSplits;
@@ -372,8 +379,17 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
       a.inline_seq[j] = seq_ids ? seq_ids[b] : b;
       a.inline_row[j] = b;
     }
-  } else if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, &a.rows, error_msg)) {
-    return rc;
+  } else {
+    // lengths and slots of a larger batch go up through the pinned ring: a copy and, when the ring wraps, a wait
+    // on the host - neither can be part of a stream capture
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    HIP_OR_RETURN(hipStreamIsCapturing(h->stream, &capturing));
+    if (capturing != hipStreamCaptureStatusNone)
+      return fail(error_msg, MI355_ATTN_FAILED_PRECONDITION,
+                  "decode of %d sequences while the stream is being captured: more than %d sequences per call need "
+                  "an upload that a capture cannot hold (capture calls of up to %d sequences)",
+                  batch, kInlineItems, kInlineItems);
+    if (int rc = upload_items(h, seq_ids, kv_lens, batch, &a.kv_lens, &a.seq_ids, &a.rows, error_msg)) return rc;
   }
   a.q = dq;
   a.out = dout;
@@ -384,8 +400,21 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   a.max_kv_len = max_len;
   a.min_kv_len = min_len;
   fill_inline_windows(h, &a);
+  bool scratch_fence = false;
+  if (no_alloc && num_splits > 1) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    HIP_OR_RETURN(hipStreamIsCapturing(h->stream, &capturing));
+    scratch_fence = capturing == hipStreamCaptureStatusNone;
+    if (scratch_fence && g_scratch_used[h->device] && g_scratch_stream[h->device] != h->stream)
+      HIP_OR_RETURN(hipStreamWaitEvent(h->stream, g_scratch_done[h->device], 0));
+  }
   HIP_OR_RETURN(launch_decode(a, h->cfg.kv_dtype, h->cfg.io_dtype, h->tuning, h->stream,
                               h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr));
+  if (scratch_fence) {
+    HIP_OR_RETURN(hipEventRecord(g_scratch_done[h->device], h->stream));
+    g_scratch_stream[h->device] = h->stream;
+    g_scratch_used[h->device] = true;
+  }
   h->timed = h->timing;
   if (new_rows)
     for (int b = 0; b < batch; ++b) note_rows_written(h, layer_begin, seq_ids ? seq_ids[b] : b, kv_lens[b] - 1, 1);
@@ -602,6 +631,9 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
       return bail(MI355_ATTN_INTERNAL, "hipGetSymbolAddress(scratch)", e);
     g_scratch_ptr[h->device] = p;
   }
+  if (!g_scratch_done[h->device] &&
+      (e = hipEventCreateWithFlags(&g_scratch_done[h->device], hipEventDisableTiming)) != hipSuccess)
+    return bail(MI355_ATTN_INTERNAL, "hipEventCreate", e);
   if (c->own_stream) {
     if ((e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking)) != hipSuccess)
       return bail(MI355_ATTN_INTERNAL, "hipStreamCreate", e);
@@ -676,6 +708,12 @@ void mi355_attn_destroy(mi355_attn* h) {
     if (ev) (void)hipEventDestroy(ev);
   if (h->ev0) (void)hipEventDestroy(h->ev0);
   if (h->ev1) (void)hipEventDestroy(h->ev1);
+  if (h->device < kMaxDevices && g_scratch_stream[h->device] == h->stream && g_scratch_used[h->device]) {
+    // (the stream was synchronised above: its last use of the shared workspace is over, and a later stream
+    // that happens to get the same address must not be taken for it)
+    g_scratch_used[h->device] = false;
+    g_scratch_stream[h->device] = nullptr;
+  }
   if (h->own_stream && h->stream) (void)hipStreamDestroy(h->stream);
   delete h;
 }

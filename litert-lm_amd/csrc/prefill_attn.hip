@@ -1346,26 +1346,28 @@ void release_plan_slot(PrefillPlans* p, int s) {
   p->valid[s] = false;
 }
 
-// Device copy of the plan for this launch shape: a cached one, or a new one built into the next slot and copied
-// on `stream` ahead of the launch.
+// Device copy of the plan for this launch shape: a cached one, or a new one built into the least recently used
+// slot that no captured graph holds and copied on `stream` ahead of the launch. *slot_out stays -1 when this
+// launch cannot have a plan: the shape is new and the stream is being captured (building one needs a copy and a
+// wait that a capture cannot hold), or every slot belongs to a captured graph. The caller then runs the kernel
+// that needs no plan.
 hipError_t plan_for(const PrefillArgs& a, int hpb, int wgs, int cus, PrefillPlans* p, hipStream_t stream, int* slot_out) {
+  *slot_out = -1;
   const int64_t key[8] = {a.layer_begin, a.n_layers, a.q_pos0, a.n, a.kchunk, wgs, hpb, a.seq};
   for (int s = 0; s < PrefillPlans::kSlots; ++s)
     if (p->valid[s] && std::equal(key, key + 8, p->key[s])) {
+      p->last_use[s] = ++p->clock;
       *slot_out = s;
       return hipSuccess;
     }
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   hipError_t e = hipStreamIsCapturing(stream, &capturing);
   if (e != hipSuccess) return e;
-  if (capturing != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;  // run the shape once before capturing it
+  if (capturing != hipStreamCaptureStatusNone) return hipSuccess;
   int s = -1;
-  for (int k = 0; k < PrefillPlans::kSlots && s < 0; ++k) {
-    const int cand = (p->next + k) % PrefillPlans::kSlots;
-    if (!p->pinned[cand]) s = cand;
-  }
-  if (s < 0) return hipErrorOutOfMemory;  // every slot belongs to a captured graph
-  p->next = (s + 1) % PrefillPlans::kSlots;
+  for (int k = 0; k < PrefillPlans::kSlots; ++k)
+    if (!p->pinned[k] && (s < 0 || p->last_use[k] < p->last_use[s])) s = k;
+  if (s < 0) return hipSuccess;  // every slot belongs to a captured graph
   if (!p->used[s] && (e = hipEventCreateWithFlags(&p->used[s], hipEventDisableTiming)) != hipSuccess) return e;
   if ((e = hipEventSynchronize(p->used[s])) != hipSuccess) return e;  // the last launch that read this slot is over
   p->valid[s] = false;
@@ -1383,6 +1385,7 @@ hipError_t plan_for(const PrefillArgs& a, int hpb, int wgs, int cus, PrefillPlan
   if (e != hipSuccess) return e;
   std::copy(key, key + 8, p->key[s]);
   p->valid[s] = true;
+  p->last_use[s] = ++p->clock;
   *slot_out = s;
   return hipSuccess;
 }
@@ -1461,16 +1464,25 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
   b.rows16 = a.rows16 < 0 ? (all_items >= 2L * cus ? 1 : 0) : a.rows16;
   // (the planned kernel needs the host's copy of the windows, and a plan of bounded size)
   if (b.rows16 == 1 && (!a.host_window || all_items > kPlanMaxItems)) b.rows16 = 0;
-  const int slots = b.rows16 == 1 ? 2 * cus : cus;
-  int wgs = all_items < slots ? (int)all_items : slots;
-  if (a.max_workgroups > 0 && a.max_workgroups < wgs) wgs = a.max_workgroups;
-  const dim3 grid(wgs, 1, 1);
+  auto workgroups = [&]() {
+    const int slots = b.rows16 == 1 ? 2 * cus : cus;
+    int w = all_items < slots ? (int)all_items : slots;
+    if (a.max_workgroups > 0 && a.max_workgroups < w) w = a.max_workgroups;
+    return w;
+  };
+  int wgs = workgroups();
   int plan_slot = -1;
   if (b.rows16 == 1) {
     hipError_t pe = plan_for(a, hpb, wgs, cus, plans, stream, &plan_slot);
     if (pe != hipSuccess) return pe;
-    b.plan = plans->d_words[plan_slot];
+    if (plan_slot >= 0) {
+      b.plan = plans->d_words[plan_slot];
+    } else {  // no plan to be had for this launch (see plan_for): the kernel that draws its work from queues
+      b.rows16 = 0;
+      wgs = workgroups();
+    }
   }
+  const dim3 grid(wgs, 1, 1);
   hipError_t err = hpb == 4   ? launch_hpb<DT, OUT, D, 4>(b, grid, stream, ev0, ev1)
                    : hpb == 2 ? launch_hpb<DT, OUT, D, 2>(b, grid, stream, ev0, ev1)
                               : launch_hpb<DT, OUT, D, 1>(b, grid, stream, ev0, ev1);
