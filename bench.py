@@ -92,6 +92,23 @@ def kernel_ms(torch, handle, step_fn, first, bursts=6, burst=32):
     return total / bursts, span / bursts
 
 
+def read_floor_ms(torch, at, nbytes, workgroups, waves, cache_bytes, bursts=4, burst=16):
+    """Duration (dispatch stamps) of a launch that only streams `nbytes` of the handle's cache with the decode
+    kernel's load pattern through `workgroups` x `waves` waves (mi355_attn_stream_probe), rotating through the
+    cache so that nothing is resident: the floor a decode launch of those bytes and that shape is priced against."""
+    span = (nbytes // (workgroups * waves) + 32767) // 32768 * 32768 * workgroups * waves
+    slots = max(1, cache_bytes // span)
+    at.set_timing(True)
+    total, i = 0.0, 0
+    for _ in range(bursts):
+        for _ in range(burst):
+            at.stream_probe((i % slots) * span, nbytes, workgroups, waves)
+            i += 1
+        total += at.last_kernel_ms()
+    at.set_timing(False)
+    return total / bursts
+
+
 def load_traffic(key):
     """HBM bytes per launch of a benchmarked kernel as last measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
     (each scaled by what the same counter reads for a plain copy of known size): profiles/traffic.json holds the
@@ -137,6 +154,7 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
         # algorithmic bytes: K and V once, Q and O once (no partials, no padding)
         per_layer = ctx * hkv * D * 2 * 2 + 2 * hq * D * 2
         step_bytes = per_layer * layers
+        floor_ms = read_floor_ms(torch, at, step_bytes, layers * hkv * splits, 1, at.cache_bytes)
 
         def step1(i):  # single layer, cache resident: latency figure only
             at.decode(0, lens, q[0, 0], out[0, 0], num_splits=splits, batch=1)
@@ -195,7 +213,7 @@ def bench_decode_c3(A, torch, steps, warmup, layers=30, rotation=4, splits=16, c
         torch.cuda.synchronize()
         at.close()
     return {"sec_per_step": sec, "timed_steps": timed, "kernel_ms": kms, "burst_ms_per_step": burst_ms,
-            "sustained_sec_per_step": sec_long, "sustained_steps": timed_long,
+            "sustained_sec_per_step": sec_long, "sustained_steps": timed_long, "floor_ms": floor_ms,
             "step_bytes": step_bytes, "layers": layers, "single_layer_latency_us": lat * 1e6,
             "tokens_per_s": 1.0 / sec, "graph": graph}
 
@@ -229,10 +247,17 @@ def bench_decode_batch(A, torch, name, kv, lens, steps, warmup, rotation, splits
     kms, _ = kernel_ms(torch, at, step, 0, bursts=4, burst=16 if layers == 1 else 4)
     esz = 1 if kv == A.I8 else 2
     nbytes = layers * (sum(lens) * hkv * D * 2 * esz + 2 * B * hq * D * 2 + (B * 2 * hkv * D * 4 if kv == A.I8 else 0))
+    # the floor: the same bytes through as many one-wave workgroups as the launch has partitions that hold keys
+    out_row = {"workload": name, "ms_per_step": sec * 1e3, "timed_steps": timed, "kernel_ms": kms, "bytes": nbytes,
+               "GBps": nbytes / sec / 1e9, "kernel_GBps": nbytes / (kms * 1e-3) / 1e9,
+               "frac_of_hbm_peak": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tokens_per_s": B / sec}
+    if layers == 1 and splits > 0:
+        per = -(-(-(-max(lens) // splits)) // 64) * 64
+        wgs = sum(-(-n // per) for n in lens) * hkv
+        floor = read_floor_ms(torch, at, nbytes, wgs, 1, at.cache_bytes)
+        out_row.update({"read_floor_ms": floor, "frac_of_read_floor": floor / kms, "read_floor_workgroups": wgs})
     at.close()
-    return {"workload": name, "ms_per_step": sec * 1e3, "timed_steps": timed, "kernel_ms": kms, "bytes": nbytes,
-            "GBps": nbytes / sec / 1e9, "kernel_GBps": nbytes / (kms * 1e-3) / 1e9,
-            "frac_of_hbm_peak": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tokens_per_s": B / sec}
+    return out_row
 
 
 def bench_decode_c1(A, torch, steps, warmup):
@@ -548,6 +573,10 @@ def main():
             "algorithmic_bytes_per_launch": dec["step_bytes"],
             "avg_kernel_us": round(dec["kernel_ms"] * 1e3, 2),
             "us_per_step_of_the_same_bursts": round(dec["burst_ms_per_step"] * 1e3, 2),
+            "read_floor_us": round(dec["floor_ms"] * 1e3, 2),
+            "frac_of_read_floor": round(dec["floor_ms"] / dec["kernel_ms"], 4),
+            "read_floor_is": "a launch of the same shape (960 one-wave workgroups) that only streams the same number of "
+                             "bytes with the kernel's load pattern (mi355_attn_stream_probe), same stamps",
         },
         "decode_graph": dec["graph"],
     }

@@ -287,6 +287,20 @@ int mi355_attn_prefill_plan_probe(int32_t n_layers, int32_t n, int32_t q_pos0, i
                                   int32_t* items_off_home);
 
 /*
+ * Measurement aid, no counterpart in the reference: streams `bytes` of the KV
+ * cache, starting `offset` bytes into it, through `workgroups` workgroups of
+ * `waves` waves with the decode kernel's load pattern (non-temporal 16-byte
+ * loads, 32 KiB per wave in flight) and does nothing with the data. With
+ * mi355_attn_set_timing on, mi355_attn_last_kernel_ms then returns the floor
+ * for a decode launch of that many bytes and that launch shape: dispatch,
+ * first-load latency and the memory's rate, no arithmetic. The cache is not
+ * changed. kOutOfRange when the shares (rounded up to whole 32 KiB pieces per
+ * wave) would pass the end of the cache.
+ */
+int mi355_attn_stream_probe(mi355_attn* handle, uint64_t offset, uint64_t bytes, int32_t workgroups, int32_t waves,
+                            char** error_msg);
+
+/*
  * Forgets the rows of sequence `seq` (seq < 0: all). Like
  * LlmLiteRtCompiledModelExecutor::Reset
  * (llm_litert_compiled_model_executor.cc:568-574) the cache memory itself is

@@ -93,6 +93,7 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_decode_noalloc.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, i32, errp]
     L.mi355_attn_decode_step.argtypes = [vp, i32, i32p, i32p, i32, vp, vp, vp, vp, i32, errp]
     L.mi355_attn_decode_layers.argtypes = [vp, i32, i32, i32p, i32p, i32, vp, vp, i32, errp]
+    L.mi355_attn_stream_probe.argtypes = [vp, ctypes.c_uint64, ctypes.c_uint64, i32, i32, errp]
     L.mi355_attn_reset.argtypes = [vp, i32, errp]
     L.mi355_attn_sync.argtypes = [vp, errp]
     L.mi355_attn_stream.argtypes = [vp]
@@ -105,7 +106,7 @@ def lib() -> ctypes.CDLL:
     L.mi355_attn_cache_bytes.restype = ctypes.c_uint64
     L.mi355_attn_version.restype = ctypes.c_char_p
     for name in ("create", "kv_append", "kv_set_scales", "kv_read", "set_layer_transform", "pre_attention", "prefill",
-                 "prefill_layers", "decode", "decode_layers", "decode_step", "decode_noalloc", "prefill_plan_probe",
+                 "prefill_layers", "decode", "decode_layers", "decode_step", "decode_noalloc", "prefill_plan_probe", "stream_probe",
                  "reset", "sync", "set_timing", "set_option"):
         getattr(L, "mi355_attn_" + name).restype = c
     _lib = L
@@ -265,6 +266,11 @@ class Attn:
         err = ctypes.c_void_p()
         _check(lib().mi355_attn_decode_noalloc(self._h, layer, sids, lens, batch, _ptr(q), _ptr(out), num_splits,
                                                ctypes.byref(err)), err)
+
+    def stream_probe(self, offset, nbytes, workgroups, waves):
+        """mi355_attn_stream_probe: a read of `nbytes` of the cache in the decode kernel's load pattern, nothing else."""
+        err = ctypes.c_void_p()
+        _check(lib().mi355_attn_stream_probe(self._h, offset, nbytes, workgroups, waves, ctypes.byref(err)), err)
 
     # -- control
     def reset(self, seq=-1):

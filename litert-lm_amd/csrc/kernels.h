@@ -70,6 +70,12 @@ hipError_t launch_prefill(const PrefillArgs& args, int kv_dtype, int io_dtype, P
 hipError_t launch_kv_append(const KvCopyArgs& args, hipStream_t stream);
 hipError_t launch_kv_read(const KvCopyArgs& args, hipStream_t stream);
 
+// Streams `bytes` of the cache from `offset` on with the decode kernel's load pattern and nothing else (the floor a
+// decode launch of that many bytes and that shape is priced against); `sink` is one device word that is never
+// written in practice. hipErrorInvalidValue when the share of the last wave would pass the end of the cache.
+hipError_t launch_stream_probe(const uint8_t* cache, int64_t cache_bytes, int64_t offset, int64_t bytes, int workgroups,
+                               int waves, uint32_t* sink, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1);
+
 // Norm + rotary embedding of n new rows, query written out, key / value rows
 // written into the cache planes (quantised for an int8 cache).
 hipError_t launch_pre_attention(const PreAttentionArgs& args, int kv_dtype, int io_dtype, hipStream_t stream,

@@ -5,6 +5,7 @@
 // compiled_model_.Run (cache tensors are inputs and outputs of every
 // signature, runtime/executor/llm_litert_compiled_model_executor.cc:733-757).
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include "attn_params.h"
 #include "kernels.h"
@@ -77,7 +78,38 @@ hipError_t launch_copy(const KvCopyArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Reads `bytes` of the cache and does nothing with them: `workgroups` x `waves` waves, each streaming a contiguous
+// share with the decode kernel's load pattern (non-temporal 16-byte loads, 32 KiB per wave in flight). The time of
+// this launch is the floor for a decode launch of the same bytes and shape: dispatch, first-load latency and the
+// memory's own rate, no arithmetic, no partial results.
+__global__ void stream_probe_kernel(const uint8_t* src, int64_t per_wave, uint32_t* sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const uint8_t* p = src + wave * per_wave + lane * 16;
+  u4 acc = {0, 0, 0, 0};
+  for (int64_t off = 0; off < per_wave; off += 32768) {
+    u4 r[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) r[i] = load_stream16(p + off + i * 1024);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) acc ^= r[i];
+  }
+  // (the zero-initialised cache and random rows never xor to this word in every lane; the store keeps the loads alive)
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u && lane == 63) sink[0] = 1;
+}
+
 }  // namespace
+
+hipError_t launch_stream_probe(const uint8_t* cache, int64_t cache_bytes, int64_t offset, int64_t bytes, int workgroups,
+                               int waves, uint32_t* sink, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  if (workgroups < 1 || waves < 1 || waves > 16 || bytes < 1 || offset < 0) return hipErrorInvalidValue;
+  const int64_t nwaves = (int64_t)workgroups * waves;
+  const int64_t per_wave = (bytes / nwaves + 32767) / 32768 * 32768;
+  if (offset % 16 || offset + per_wave * nwaves > cache_bytes) return hipErrorInvalidValue;  // every load inside the cache
+  hipExtLaunchKernelGGL(stream_probe_kernel, dim3(workgroups), dim3(waves * 64), 0, stream, ev0, ev1, 0, cache + offset,
+                        per_wave, sink);
+  return hipGetLastError();
+}
 
 hipError_t launch_kv_append(const KvCopyArgs& a, hipStream_t stream) { return launch_copy<true>(a, stream); }
 hipError_t launch_kv_read(const KvCopyArgs& a, hipStream_t stream) { return launch_copy<false>(a, stream); }

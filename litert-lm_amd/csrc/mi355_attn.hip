@@ -659,7 +659,7 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
   if ((e = hipMemcpyAsync(h->d_window, h->window.data(), sizeof(int32_t) * c->num_layers, hipMemcpyHostToDevice,
                           h->stream)) != hipSuccess)
     return bail(MI355_ATTN_INTERNAL, "window upload", e);
-  if ((e = hipMalloc(&h->d_sched, sizeof(int32_t) * kPrefillSchedInts)) != hipSuccess)
+  if ((e = hipMalloc(&h->d_sched, sizeof(int32_t) * (kPrefillSchedInts + 1))) != hipSuccess)  // (+ the stream probe's sink word)
     return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "prefill queue counters", e);
   h->transform.assign(c->num_layers, mi355_attn::LayerTransform{});
   const size_t transform_bytes = sizeof(float) * (size_t)c->num_layers * transform_floats(c->head_dim);
@@ -964,6 +964,25 @@ int mi355_attn_decode_noalloc(mi355_attn* h, int32_t layer, const int32_t* seq_i
                               int32_t batch, const void* q, void* out, int32_t num_splits, char** error_msg) {
   static_assert(kNoAllocHeadDim == 256, "the workspace is laid out for the one head_dim the library builds");
   return decode_impl(h, layer, 1, seq_ids, kv_lens, batch, q, out, num_splits, error_msg, /*no_alloc=*/true);
+}
+
+int mi355_attn_stream_probe(mi355_attn* h, uint64_t offset, uint64_t bytes, int32_t workgroups, int32_t waves,
+                            char** error_msg) {
+  if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
+  if (workgroups < 1 || waves < 1 || waves > 16 || bytes < 1)
+    return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "workgroups >= 1, 1 <= waves <= 16 and bytes >= 1");
+  HIP_OR_RETURN(hipSetDevice(h->device));
+  hipError_t e = launch_stream_probe(h->cache, (int64_t)h->cache_bytes, (int64_t)offset, (int64_t)bytes, workgroups, waves,
+                                     reinterpret_cast<uint32_t*>(h->d_sched) + kPrefillSchedInts, h->stream,
+                                     h->timing ? h->ev0 : nullptr, h->timing ? h->ev1 : nullptr);
+  if (e == hipErrorInvalidValue)
+    return fail(error_msg, MI355_ATTN_OUT_OF_RANGE,
+                "%llu bytes from offset %llu in %d x %d shares of whole 32 KiB pieces do not fit the cache (%llu bytes), or "
+                "the offset is not a multiple of 16",
+                (unsigned long long)bytes, (unsigned long long)offset, workgroups, waves, (unsigned long long)h->cache_bytes);
+  HIP_OR_RETURN(e);
+  h->timed = h->timing;
+  return MI355_ATTN_OK;
 }
 
 int mi355_attn_reset(mi355_attn* h, int32_t seq, char** error_msg) {

@@ -1483,9 +1483,13 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
     }
   }
   const dim3 grid(wgs, 1, 1);
+#ifdef MI355_PREFILL_ONE_SHAPE  // (development builds: one instantiation compiles in a tenth of the time)
+  hipError_t err = hpb == 4 ? launch_hpb<DT, OUT, D, 4>(b, grid, stream, ev0, ev1) : hipErrorInvalidValue;
+#else
   hipError_t err = hpb == 4   ? launch_hpb<DT, OUT, D, 4>(b, grid, stream, ev0, ev1)
                    : hpb == 2 ? launch_hpb<DT, OUT, D, 2>(b, grid, stream, ev0, ev1)
                               : launch_hpb<DT, OUT, D, 1>(b, grid, stream, ev0, ev1);
+#endif
   if (err == hipSuccess && plan_slot >= 0) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     err = hipStreamIsCapturing(stream, &capturing);
@@ -1602,10 +1606,14 @@ bool prefill_supported(int kv_dtype, int io_dtype, int head_dim) {
 
 hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, PrefillPlans* plans, hipStream_t stream,
                           hipEvent_t ev0, hipEvent_t ev1) {
+#ifdef MI355_PREFILL_ONE_SHAPE
+  if (kv_dtype == kBF16 && io_dtype == kBF16) return launch_typed<kBF16, kBF16, 256>(a, plans, stream, ev0, ev1);
+#else
   if (kv_dtype == kF16 && io_dtype == kF16) return launch_typed<kF16, kF16, 256>(a, plans, stream, ev0, ev1);
   if (kv_dtype == kF16 && io_dtype == kF32) return launch_typed<kF16, kF32, 256>(a, plans, stream, ev0, ev1);
   if (kv_dtype == kBF16 && io_dtype == kBF16) return launch_typed<kBF16, kBF16, 256>(a, plans, stream, ev0, ev1);
   if (kv_dtype == kBF16 && io_dtype == kF32) return launch_typed<kBF16, kF32, 256>(a, plans, stream, ev0, ev1);
+#endif
   return hipErrorInvalidValue;
 }
 

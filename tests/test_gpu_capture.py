@@ -135,3 +135,27 @@ def test_noalloc_calls_on_two_streams_are_ordered_by_the_library():
     finally:
         at1.close()
         at2.close()
+
+
+def test_stream_probe_reads_without_touching_the_cache_and_checks_its_range():
+    with A.Attn(2, 4, 1, D, 1024, 2, A.F16, A.F16, stream=torch.cuda.current_stream().cuda_stream) as at:
+        k, v = rnd(3, 1024, 1, D), rnd(4, 1024, 1, D)
+        at.kv_append(1, 1, 0, k, v)
+        total = at.cache_bytes  # 2 layers x 2 sequences x 2 planes x 512 KiB = 4 MiB
+        assert total == 2 * 2 * 2 * 1024 * D * 2
+        at.set_timing(True)
+        at.stream_probe(0, total, 32, 1)
+        ms = at.last_kernel_ms()
+        at.stream_probe(32768, total // 2, 8, 4)
+        at.set_timing(False)
+        assert ms > 0
+        for off, nbytes, wgs, waves, code in ((0, total + 32 * 32768, 32, 1, A.OUT_OF_RANGE), (8, 1024, 1, 1, A.OUT_OF_RANGE),
+                                              (total - 1024, 32768, 1, 1, A.OUT_OF_RANGE), (0, 1024, 0, 1, A.INVALID_ARGUMENT),
+                                              (0, 1024, 1, 17, A.INVALID_ARGUMENT)):
+            with pytest.raises(A.AttnError) as e:
+                at.stream_probe(off, nbytes, wgs, waves)
+            assert e.value.code == code, (off, nbytes, wgs, waves)
+        ko, vo = torch.zeros_like(k), torch.zeros_like(v)
+        at.kv_read(1, 1, 0, 1024, ko, vo)
+        torch.cuda.synchronize()
+        assert torch.equal(ko, k) and torch.equal(vo, v)
