@@ -334,6 +334,43 @@ def bench_prefill_c2(A, torch, steps, warmup, layers=26, n=1024, half=False, by_
             "dense_counted_TFLOPs": layers * 4 * hq * D * n * n / sec / 1e12}
 
 
+def bench_prefill_int8(A, torch, steps, warmup, layers, n, q_pos0, hq, hkv, windows=None):
+    """Prefill over an int8 cache: the call as it runs by default (the planes it reads staged as half planes, then
+    the matrix-core kernels of a half cache) beside the row-wise path (every query row a decode item, converted in
+    registers). Whole calls, staging included; the FLOPs are those of the visible (query, key) pairs."""
+    windows = windows or [0] * layers
+    ctx = q_pos0 + n
+    stream = torch.cuda.current_stream().cuda_stream
+    at = A.Attn(layers, hq, hkv, D, ctx, 1, A.I8, A.F16, layer_window=windows, stream=stream)
+    g = torch.Generator(device="cuda:0").manual_seed(0xC0FFEE + 9)
+    for layer in range(layers):
+        k = torch.randint(-127, 128, (ctx, hkv, D), generator=g, device="cuda:0", dtype=torch.int8)
+        v = torch.randint(-127, 128, (ctx, hkv, D), generator=g, device="cuda:0", dtype=torch.int8)
+        at.kv_append(layer, 0, 0, k, v)
+        at.kv_set_scales(layer, 0, torch.rand((hkv, D), generator=g, device="cuda:0") * 0.02 + 0.005,
+                         torch.rand((hkv, D), generator=g, device="cuda:0") * 0.02 + 0.005)
+    q = torch.randn((layers, n, hq, D), device="cuda:0").half()
+    out = torch.empty_like(q)
+
+    def step(i):
+        at.prefill(0, 0, q_pos0, n, q, out, n_layers=layers)
+
+    flops = 0
+    for w in windows:
+        pairs = sum(min(q_pos0 + i + 1, w) if w > 0 else q_pos0 + i + 1 for i in range(n))
+        flops += 4 * hq * D * pairs
+    sec, timed = time_steps(torch, step, steps, warmup)
+    kms, _ = kernel_ms(torch, at, step, 0)
+    at.set_option("rowwise_prefill", 1)
+    sec_row, _ = time_steps(torch, step, max(3, steps // 4), 2)
+    kms_row, _ = kernel_ms(torch, at, step, 0, bursts=2, burst=8)
+    at.close()
+    return {"ms_per_step": sec * 1e3, "timed_steps": timed, "flops": flops, "TFLOPs": flops / sec / 1e12,
+            "call_us_device": kms * 1e3, "device_TFLOPs": flops / (kms * 1e-3) / 1e12,
+            "rowwise_ms_per_step": sec_row * 1e3, "rowwise_TFLOPs": flops / sec_row / 1e12,
+            "rowwise_kernel_us": kms_row * 1e3, "rowwise_kernel_TFLOPs": flops / (kms_row * 1e-3) / 1e12}
+
+
 def gemm_probe(torch, n=8192, reps=20):
     """Dense bf16 GEMM through the vendor library: what the matrix cores of this
     very card sustain next to the published peak the roofline is priced on."""
@@ -628,6 +665,32 @@ def main():
                                             "small launches use (the default picks the 16x16x32 kernel here)",
             "value": round(pre32["TFLOPs"], 2), "unit": "TFLOP/s", "kernel_TFLOPs": round(pre32["kernel_TFLOPs"], 2),
             "frac_of_mfma_peak": round(pre32["frac_of_mfma_peak"], 4), "avg_kernel_us": round(pre32["kernel_ms"] * 1e3, 2)}
+        i8_rows = []
+        for name, kw in (("one layer, Hq8/Hkv2 (config 5's heads), rows 0..1023 of a sequence",
+                          dict(layers=1, n=1024, q_pos0=0, hq=8, hkv=2)),
+                         ("one layer, Hq8/Hkv2, rows 3072..4095 of a 4096-token sequence",
+                          dict(layers=1, n=1024, q_pos0=3072, hq=8, hkv=2)),
+                         ("26 layers x 1024 tokens, Hq4/Hkv1, 22 local(W=512)+4 global (config 2's shape on an int8 cache)",
+                          dict(layers=26, n=1024, q_pos0=0, hq=4, hkv=1,
+                               windows=[0 if (l + 1) % 6 == 0 else 512 for l in range(26)]))):
+            r = bench_prefill_int8(A, torch, few, fw, **kw)
+            log(f"[bench] prefill int8, {name}: {r['ms_per_step'] * 1e3:.1f} us/call = {r['TFLOPs']:.1f} TFLOP/s "
+                f"(device time {r['call_us_device']:.1f} us = {r['device_TFLOPs']:.1f} TFLOP/s); row-wise path "
+                f"{r['rowwise_ms_per_step'] * 1e3:.1f} us/call = {r['rowwise_TFLOPs']:.2f} TFLOP/s")
+            i8_rows.append({"workload": name, "unit": "TFLOP/s", "value": round(r["TFLOPs"], 2),
+                            "us_per_call": round(r["ms_per_step"] * 1e3, 2),
+                            "device_us_per_call": round(r["call_us_device"], 2),
+                            "device_TFLOPs": round(r["device_TFLOPs"], 2),
+                            "frac_of_mfma_peak": round(r["device_TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                            "rowwise_path": {"value": round(r["rowwise_TFLOPs"], 3), "us_per_call": round(r["rowwise_ms_per_step"] * 1e3, 2),
+                                             "kernel_us": round(r["rowwise_kernel_us"], 2),
+                                             "kernel_TFLOPs": round(r["rowwise_kernel_TFLOPs"], 3)}})
+        result["prefill_int8"] = {
+            "what": "prefill over an int8 cache, fp16 activations. value: whole calls back to back (query staging, "
+                    "the planes' conversion to half planes, attention); device_us_per_call: from the start of the first "
+                    "of those launches to the end of the attention kernel; rowwise_path: the same call with option "
+                    "rowwise_prefill=1 (every query row a decode item, int8 converted in registers)",
+            "rows": i8_rows}
         probe = gemm_probe(torch)
         log(f"[bench] vendor bf16 GEMM 8192^3: {probe:.0f} TFLOP/s")
         result["mfma_peak_probe"] = {"what": "torch.matmul bf16 8192x8192x8192 (hipBLASLt)", "TFLOPs": round(probe, 1),

@@ -32,6 +32,16 @@
  * are rounded to it (nearest even) on the way in (a prefill call does so in a
  * pass of its own over the query rows), products accumulate in float32 and
  * the output is written in io_dtype from those sums.
+ * An int8 cache enters the matrix cores as IEEE half values. Decode converts in
+ * registers (K scales folded into the queries, V scales applied to the sums). A
+ * prefill call of 16 rows or more first turns the planes it reads into half
+ * planes in a staging area of the handle (2 bytes per cache byte of the layers of
+ * a pass, grown on demand up to "prefill_i8_stage_mib"; the call runs in passes
+ * over as many layers as fit), V as half(value x scale), K as the values
+ * themselves with the scales folded into float32 / bfloat16 queries on their way
+ * to half, or as half(value x scale) under half queries, which are read as they
+ * are; smaller calls, and calls that would have to allocate while the stream is
+ * being captured, run row by row through the decode kernel.
  * A bfloat16 cache keeps its K planes in bfloat16 and its V planes as IEEE half
  * values, so that the probabilities multiply V with 11 significant bits on the
  * fp16 matrix-core path: a bfloat16 value v is stored without loss for
@@ -329,7 +339,12 @@ float mi355_attn_last_kernel_ms(mi355_attn* handle);
  *   "decode_waves"     1, 2 or 4 waves per decode workgroup, 0 (default) = chosen
  *                      from the number of workgroups of the launch
  *   "rowwise_prefill"  0/1 run prefill row by row through the decode kernel
- *                      (the only path for fp32 and int8 caches)
+ *                      (the only path for an fp32 cache)
+ *   "prefill_i8_min_rows" int8 cache: prefill calls of fewer rows run row by row
+ *                      (default 16)
+ *   "prefill_i8_stage_mib" int8 cache: limit of the staging area for half planes,
+ *                      MiB (default 2048; one layer's planes are staged even when
+ *                      they exceed it)
  *   "prefill_workgroups" upper bound of the persistent workgroups of the prefill
  *                      kernel, 0 (default) = one per compute unit
  *   "prefill_rows16"   which of the two prefill kernels runs: 1 the one on 16x16x32 MFMAs

@@ -143,7 +143,11 @@ MI355_HD void decode_visible_range(int kv_len, int window, int* vlo, int* start)
 struct PrefillArgs {
   const void* q;   // [n_layers][n][hq][D], io type
   void* out;
-  void* q_stage;   // float32 activations over a 16-bit cache: room for the queries in the cache's type (else unused)
+  void* q_stage;   // room for the call's queries in the type the matrix cores take, 2 bytes per element, where that is
+                   // not the activations' type: float32 activations, bfloat16 activations over an int8 cache
+  int32_t q_staged;        // != 0: q is of the kernels' type already (set by the int8 path for the kernels it runs)
+  void* kv_stage;          // int8 cache: room for the half planes the call reads (prefill_i8_stage_bytes)
+  int64_t kv_stage_bytes;
   const uint8_t* cache;
   const float* scales;
   const int32_t* layer_window;

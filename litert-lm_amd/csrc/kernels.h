@@ -21,6 +21,8 @@ hipError_t launch_decode(const DecodeArgs& args, int kv_dtype, int io_dtype, con
                          hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1);
 
 bool prefill_supported(int kv_dtype, int io_dtype, int head_dim);
+// Bytes of half planes that a prefill over an int8 cache stages for `n_layers` layers of a call ending at row `end`.
+int64_t prefill_i8_stage_bytes(const CacheGeom& geom, int n_layers, int end);
 
 // Key split of a prefill launch (PrefillArgs::kchunk / smax): none (kchunk 0) unless the launch has
 // fewer work items than three quarters of the compute units; then at most 8 items per tile of at

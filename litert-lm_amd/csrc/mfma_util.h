@@ -69,6 +69,20 @@ __device__ __forceinline__ void cvt_i8x16_to_h8x2(u4 w, h8& lo, h8& hi) {
   hi = bit_cast<h8>(b) - bias;
 }
 
+// 8 two's-complement int8 (8 bytes) -> one h8, element order kept (half of cvt_i8x16_to_h8x2).
+__device__ __forceinline__ h8 cvt_i8x8_to_h8(u2 w) {
+  unsigned o[4];
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const unsigned x = w[d] ^ 0x80808080u;
+    o[2 * d] = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+    o[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+  }
+  const h8 bias = {1152, 1152, 1152, 1152, 1152, 1152, 1152, 1152};
+  const u4 a = {o[0], o[1], o[2], o[3]};
+  return bit_cast<h8>(a) - bias;
+}
+
 // bfloat16 bits -> the IEEE half that a V plane of a bfloat16 cache stores (exact for
 // 2^-17 <= |v| <= 65504, finite values above saturate, nearest multiple of 2^-24 below), and back.
 // NaN and +-infinity pass through as NaN and +-infinity (fminf / fmaxf would turn a NaN into a bound).

@@ -94,8 +94,12 @@ struct mi355_attn {
   float* d_pf_acc = nullptr;   // prefill key split: parts of split tiles, allocated on first use
   float* d_pf_ml = nullptr;
   size_t pf_rows = 0;          // rows (of head_dim / of 2 floats) the two hold
-  void* d_q_stage = nullptr;   // prefill with float32 activations over a 16-bit cache: the queries in the cache's type
+  void* d_q_stage = nullptr;   // prefill whose queries are staged (float32 activations; bfloat16 ones over an int8 cache)
   size_t q_stage_bytes = 0;
+  void* d_kv_stage = nullptr;  // prefill over an int8 cache: the half planes of the layers of a pass
+  size_t kv_stage_bytes = 0;
+  int prefill_i8_min_rows = 16;  // int8 cache: calls of fewer rows take the row-wise path
+  int prefill_i8_stage_mib = 2048;  // int8 cache: limit of the staging area (a pass covers as many layers as fit, at least one)
   int prefill_key_split = -1;  // < 0 by rule, 0 off, > 0 key blocks per work item
   int prefill_rows16 = -1;     // which prefill kernel: 1 the one on 16x16x32 MFMAs, 0 the one on 32x32x16, < 0 by rule
   // the step before attention: per-layer constants in HBM and what is switched on
@@ -443,10 +447,42 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
   if (int rc = stage_in(h, 0, q, io_bytes, &dq, error_msg)) return rc;
   if (int rc = stage_out_begin(h, 1, out, io_bytes, &dout, error_msg)) return rc;
   hipEvent_t e0 = h->timing ? h->ev0 : nullptr, e1 = h->timing ? h->ev1 : nullptr;
-  if (prefill_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim) && !h->rowwise_prefill) {
+  bool rowwise = !prefill_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim) || h->rowwise_prefill;
+  // An int8 cache goes to the matrix cores through half planes staged per call (prefill_attn.hip): from a tile's
+  // worth of rows on, in passes of as many layers as the staging area's limit holds.
+  const bool i8 = h->cfg.kv_dtype == MI355_ATTN_I8;
+  int layers_per_pass = n_layers;
+  if (!rowwise && i8) {
+    if (n < h->prefill_i8_min_rows) {
+      rowwise = true;
+    } else {
+      const int64_t kStageMax = (int64_t)h->prefill_i8_stage_mib << 20;
+      const int64_t per_layer = prefill_i8_stage_bytes(h->geom, 1, q_pos0 + n);
+      layers_per_pass = (int)std::min<int64_t>(n_layers, std::max<int64_t>(1, kStageMax / per_layer));
+      const size_t need = (size_t)per_layer * layers_per_pass;
+      if (h->kv_stage_bytes < need) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        HIP_OR_RETURN(hipStreamIsCapturing(h->stream, &capturing));
+        if (capturing != hipStreamCaptureStatusNone) {
+          rowwise = true;  // (nothing can be allocated while a graph is recorded: the path that needs no room)
+        } else {
+          HIP_OR_RETURN(hipStreamSynchronize(h->stream));
+          if (h->d_kv_stage) HIP_OR_RETURN(hipFree(h->d_kv_stage));
+          h->d_kv_stage = nullptr;
+          h->kv_stage_bytes = 0;
+          HIP_OR_RETURN(hipMalloc(&h->d_kv_stage, need));
+          h->kv_stage_bytes = need;
+        }
+      }
+    }
+  }
+  const size_t layer_io_bytes = (size_t)n * h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
+  for (int l0 = 0; !rowwise && l0 < n_layers; l0 += layers_per_pass) {
+    const int nl = std::min(layers_per_pass, n_layers - l0);
+    hipEvent_t pe0 = l0 == 0 ? e0 : nullptr, pe1 = l0 + nl == n_layers ? e1 : nullptr;
     PrefillArgs a{};
-    a.q = dq;
-    a.out = dout;
+    a.q = static_cast<const uint8_t*>(dq) + l0 * layer_io_bytes;
+    a.out = static_cast<uint8_t*>(dout) + l0 * layer_io_bytes;
     a.cache = h->cache;
     a.scales = h->scales;
     a.layer_window = h->d_window;
@@ -454,8 +490,8 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.geom = h->geom;
     a.hq = h->cfg.num_q_heads;
     a.group = h->cfg.num_q_heads / h->cfg.num_kv_heads;
-    a.layer_begin = layer_begin;
-    a.n_layers = n_layers;
+    a.layer_begin = layer_begin + l0;
+    a.n_layers = nl;
     a.seq = seq;
     a.q_pos0 = q_pos0;
     a.n = n;
@@ -464,8 +500,8 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     a.max_workgroups = h->prefill_workgroups;
     a.rows16 = h->prefill_rows16;
     a.host_window = h->window.data();
-    if (h->cfg.io_dtype != h->cfg.kv_dtype) {
-      const size_t need = (size_t)n_layers * n * h->cfg.num_q_heads * h->cfg.head_dim * kv_size(h);
+    if (h->cfg.io_dtype != h->cfg.kv_dtype && !(i8 && h->cfg.io_dtype == MI355_ATTN_F16)) {
+      const size_t need = (size_t)nl * n * h->cfg.num_q_heads * h->cfg.head_dim * 2;
       if (h->q_stage_bytes < need) {
         HIP_OR_RETURN(hipStreamSynchronize(h->stream));
         if (h->d_q_stage) HIP_OR_RETURN(hipFree(h->d_q_stage));
@@ -476,6 +512,8 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
       }
       a.q_stage = h->d_q_stage;
     }
+    a.kv_stage = h->d_kv_stage;
+    a.kv_stage_bytes = (int64_t)h->kv_stage_bytes;
     PrefillSplit split = plan_prefill_split(a, h->prefill_key_split);
     constexpr size_t kSplitRowsMax = (size_t)256 << 10;  // 256 Ki rows = 258 MiB at head_dim 256
     if (split.kchunk > 0 && split.rows > kSplitRowsMax && h->prefill_key_split < 0) split = PrefillSplit{};
@@ -498,8 +536,9 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
       a.ws_acc = h->d_pf_acc;
       a.ws_ml = h->d_pf_ml;
     }
-    HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, &h->pf_plans, h->stream, e0, e1));
-  } else {
+    HIP_OR_RETURN(launch_prefill(a, h->cfg.kv_dtype, h->cfg.io_dtype, &h->pf_plans, h->stream, pe0, pe1));
+  }
+  if (rowwise) {
     // Row-wise path (fp32 and int8 caches): every query row is one decode item
     // whose key range ends at its own position.
     if (!decode_supported(h->cfg.kv_dtype, h->cfg.io_dtype, h->cfg.head_dim))
@@ -508,7 +547,13 @@ int prefill_impl(mi355_attn* h, int layer_begin, int n_layers, int seq, int q_po
     if (n > 65535)
       return fail(error_msg, MI355_ATTN_UNIMPLEMENTED,
                   "row-wise prefill (fp32 / int8 cache): %d rows exceed the launch grid (65535); call in chunks", n);
-    if (h->d_items_cap < (size_t)n) {
+    if (h->d_items_cap < (size_t)n) {  // (never for an int8 or float32 cache: theirs is there from the start)
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      HIP_OR_RETURN(hipStreamIsCapturing(h->stream, &capturing));
+      if (capturing != hipStreamCaptureStatusNone)
+        return fail(error_msg, MI355_ATTN_FAILED_PRECONDITION,
+                    "row-wise prefill needs its item list allocated, which cannot happen while the stream is being "
+                    "captured: run one row-wise prefill before the capture");
       HIP_OR_RETURN(hipStreamSynchronize(h->stream));
       if (h->d_items) HIP_OR_RETURN(hipFree(h->d_items));
       h->d_items = nullptr;
@@ -669,6 +714,13 @@ int mi355_attn_create(const mi355_attn_config* c, mi355_attn** out, char** error
     return bail(MI355_ATTN_INTERNAL, "layer transform clear", e);
   if ((e = hipMemsetAsync(h->d_sched, 0, sizeof(int32_t) * kPrefillSchedInts, h->stream)) != hipSuccess)
     return bail(MI355_ATTN_INTERNAL, "prefill queue clear", e);
+  if (c->kv_dtype == MI355_ATTN_I8 || c->kv_dtype == MI355_ATTN_F32) {
+    // the row-wise prefill path's item list (these caches may take that path inside a captured graph, where nothing
+    // can be allocated)
+    if ((e = hipMalloc(&h->d_items, sizeof(int32_t) * 2 * (size_t)c->max_tokens)) != hipSuccess)
+      return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "row-wise prefill items", e);
+    h->d_items_cap = c->max_tokens;
+  }
   h->ring_slot_ints = 3 * c->max_seqs;
   if ((e = hipHostMalloc(&h->h_ring, sizeof(int32_t) * h->ring_slot_ints * kRingSlots)) != hipSuccess)
     return bail(MI355_ATTN_RESOURCE_EXHAUSTED, "pinned ring", e);
@@ -696,6 +748,7 @@ void mi355_attn_destroy(mi355_attn* h) {
   if (h->d_pf_acc) (void)hipFree(h->d_pf_acc);
   if (h->d_pf_ml) (void)hipFree(h->d_pf_ml);
   if (h->d_q_stage) (void)hipFree(h->d_q_stage);
+  if (h->d_kv_stage) (void)hipFree(h->d_kv_stage);
   if (h->d_transform) (void)hipFree(h->d_transform);
   if (h->ws_acc) (void)hipFree(h->ws_acc);
   if (h->ws_ml) (void)hipFree(h->ws_ml);
@@ -1032,6 +1085,12 @@ int mi355_attn_set_option(mi355_attn* h, const char* name, int32_t value) {
   } else if (!strcmp(name, "prefill_rows16")) {
     if (value < -1 || value > 1) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_rows16 = value;
+  } else if (!strcmp(name, "prefill_i8_stage_mib")) {
+    if (value < 1) return MI355_ATTN_INVALID_ARGUMENT;
+    h->prefill_i8_stage_mib = value;
+  } else if (!strcmp(name, "prefill_i8_min_rows")) {
+    if (value < 1) return MI355_ATTN_INVALID_ARGUMENT;
+    h->prefill_i8_min_rows = value;
   } else if (!strcmp(name, "prefill_key_split")) {
     if (value < -1 || value > 4096) return MI355_ATTN_INVALID_ARGUMENT;
     h->prefill_key_split = value;

@@ -122,7 +122,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 template <int DT, int OUT, int D, int HPB, bool CAP>
 __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const PrefillArgs a) {
   using E = El<DT>;
-  using elem_t = typename E::type;
+  using out_t = typename OutEl<OUT>::type;
   using vec8 = typename E::vec8;
   constexpr int PT = 4 / HPB;            // stretches per workgroup
   constexpr int NJ = D / 16;             // K-slices of the QK^T product
@@ -610,9 +610,9 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
     for (int dp = 0; dp < NDP; ++dp) {
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
-        elem_t o[4];
+        out_t o[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) o[b] = (elem_t)(acc0[dp][4 * aa + b] * inv);
+        for (int b = 0; b < 4; ++b) o[b] = (out_t)(acc0[dp][4 * aa + b] * inv);
         *reinterpret_cast<u2*>(patch + n * kRowStride + (32 * dp + 8 * aa + 4 * hh) * 2) = *reinterpret_cast<const u2*>(o);
       }
     }
@@ -625,7 +625,7 @@ __global__ void __launch_bounds__(kWaves * 64) prefill_attn_kernel(const Prefill
       const u4 w = *reinterpret_cast<const u4*>(patch + r * kRowStride + chunk * 16);
       const int row = row_base + r;
       if (row < a.n) {
-        elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
+        out_t* orow = reinterpret_cast<out_t*>(a.out) + (((int64_t)li * a.n + row) * a.hq + head) * D;
         *reinterpret_cast<u4*>(orow + chunk * 8) = w;
       }
     }
@@ -679,6 +679,7 @@ template <int DT, int OUT, int D, int HPB, bool CAP>
 __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const PrefillArgs a) {
   using E = El<DT>;
   using elem_t = typename E::type;
+  using out_t = typename OutEl<OUT>::type;
   using vec8 = typename E::vec8;
   constexpr int PT = 4 / HPB;
   constexpr int NJ = D / 32;  // 32-channel steps of the QK^T product
@@ -1023,16 +1024,16 @@ __global__ void __launch_bounds__(kWaves16 * 64, 2) prefill_attn16_kernel(const 
           uint32_t packed[NL][2];
 #pragma unroll
           for (int db = 0; db < NL; ++db) {
-            elem_t o[4];
+            out_t o[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (elem_t)(acc[u][db][e] * inv);
+            for (int e = 0; e < 4; ++e) o[e] = (out_t)(acc[u][db][e] * inv);
             const u2 w = *reinterpret_cast<const u2*>(o);
             packed[db][0] = w[0];
             packed[db][1] = w[1];
           }
           // lanes g = 0, 2 keep tile 2k (channels 32k + 4g .. + 7), lanes g = 1, 3 tile 2k + 1 (32k + 16 + 4(g - 1) .. + 7)
           const int first = (g & 1) * 16 + (g >> 1) * 8;
-          elem_t* orow = reinterpret_cast<elem_t*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + first;
+          out_t* orow = reinterpret_cast<out_t*>(a.out) + (((int64_t)it.li * a.n + row) * a.hq + it.head) * D + first;
 #pragma unroll
           for (int k = 0; k < NL / 2; ++k) {
             const auto lo = __builtin_amdgcn_permlane16_swap(packed[2 * k][0], packed[2 * k + 1][0], false, false);
@@ -1407,7 +1408,7 @@ hipError_t launch_typed(const PrefillArgs& a, PrefillPlans* plans, hipStream_t s
   }
   PrefillArgs b = a;
   b.use_order = 0;
-  if constexpr (OUT != DT) {
+  if (OUT != DT && !a.q_staged) {
     // float32 activations: the queries go through the staging rows in the cache's type first
     if (!a.q_stage) return hipErrorInvalidValue;
     const int64_t n8 = (int64_t)a.n_layers * a.n * a.hq * D / 8;
@@ -1601,7 +1602,161 @@ PrefillSplit plan_prefill_split(const PrefillArgs& a, int option) {
 }
 
 bool prefill_supported(int kv_dtype, int io_dtype, int head_dim) {
-  return head_dim == 256 && (kv_dtype == kF16 || kv_dtype == kBF16) && (io_dtype == kv_dtype || io_dtype == kF32);
+  if (head_dim != 256) return false;
+  if (kv_dtype == kI8) return io_dtype == kF32 || io_dtype == kF16 || io_dtype == kBF16;
+  return (kv_dtype == kF16 || kv_dtype == kBF16) && (io_dtype == kv_dtype || io_dtype == kF32);
+}
+
+// ---------------------------------------------------------------------------
+// An int8 cache on the matrix cores: the planes the call reads are turned into IEEE half planes once, in a staging
+// area of the handle, and the kernels of a half cache run on those. The V planes take their scales with them
+// (half(int8 value x float32 scale of its channel)). The K scales go where they cost nothing:
+//   - float32 and bfloat16 activations pass through a conversion to half anyway, and take the scales there
+//     (half(q x scale)); the K planes are then the int8 values themselves, exact in half;
+//   - half activations are read by the attention kernel as they are (a pass over them just for the scales is 27 us
+//     of an 83 us call at 26 layers x 1,024 rows), and the K planes take the scales (half(value x scale)).
+// Either way a product of the scores has one operand rounded to half once, as in the decode kernel.
+//   Why not in the attention kernel's registers, as the decode kernel does it: there every byte is converted once;
+// here a K or V block is an operand of every query tile that sees it, so each of the workgroup's four waves would
+// convert it again for each of its tiles, ten vector instructions for every two matrix instructions of 16 cycles,
+// which bounds the kernel at half the matrix rate before the softmax is counted; and with 192 of a wave's 256
+// registers holding accumulators and queries, the converted operands and their temporaries find no room (every
+// arrangement tried spilled 30 to 150 registers, queries loaded behind the compiler's back among them).
+// Converting once per call costs three bytes of HBM traffic per cache byte, against attention work that grows
+// with the number of query rows.
+// float32 or bfloat16 queries as the halves the kernels take, with the K scales of the head's plane folded in (the
+// K planes of such a call are staged as the int8 values themselves): half(q x scale), one thread per 8 channels of
+// a query row.
+template <int IO, int D>
+__global__ void __launch_bounds__(256) stage_queries_i8_kernel(const void* __restrict__ q, _Float16* __restrict__ dst,
+                                                               const float* __restrict__ scales, CacheGeom geom, int layer_begin,
+                                                               int seq, int n, int hq, int group, int64_t pieces) {
+  static_assert(IO == kF32 || IO == kBF16, "half queries are taken as they are");
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= pieces) return;
+  constexpr int kPieces = D / 8;
+  const int d0 = 8 * (int)(i % kPieces);
+  const int64_t row = i / kPieces;  // (layer, token, head)
+  const int head = (int)(row % hq);
+  const int li = (int)(row / ((int64_t)n * hq));
+  const float* ks = scales + geom.scale_offset(layer_begin + li, seq, 0, head / group) + d0;
+  f4 x0, x1;
+  if constexpr (IO == kF32) {
+    const float* src = reinterpret_cast<const float*>(q) + row * D + d0;
+    x0 = *reinterpret_cast<const f4*>(src);
+    x1 = *reinterpret_cast<const f4*>(src + 4);
+  } else {
+    const b8 v = *reinterpret_cast<const b8*>(reinterpret_cast<const __bf16*>(q) + row * D + d0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { x0[e] = (float)v[e]; x1[e] = (float)v[4 + e]; }
+  }
+  const f4 s0 = *reinterpret_cast<const f4*>(ks), s1 = *reinterpret_cast<const f4*>(ks + 4);
+  h8 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { o[e] = (_Float16)(x0[e] * s0[e]); o[4 + e] = (_Float16)(x1[e] * s1[e]); }
+  *reinterpret_cast<h8*>(dst + row * D + d0) = o;
+}
+
+// Grid (chunks of a plane's range / 256, planes of the call): one thread per 16-byte chunk of an int8 plane, which
+// becomes two 16-byte chunks of the half plane (attn_params.h has both layouts):
+//   K: chunk c of token t (channels 16 c .. + 15) -> chunks 2 c and 2 c + 1 of the same token, tile and row;
+//   V: a chunk holds 16 tokens of one channel, slots 4 T + j of a 64-token block; slots 0..7 are the 8 slots of the
+//      same chunk position in half block 2 B, slots 8..15 those in half block 2 B + 1.
+// Blocks of 64 tokens that no query of the call sees (in front of a layer's window) are left alone.
+__global__ void __launch_bounds__(256) dequant_planes_kernel(const uint8_t* __restrict__ cache, const float* __restrict__ scales,
+                                                             CacheGeom src, uint8_t* __restrict__ staged, CacheGeom dst,
+                                                             const int32_t* __restrict__ layer_window, int layer_begin,
+                                                             int seq, int q_pos0, int64_t chunks, int scale_k) {
+  const int64_t ci = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (ci >= chunks) return;
+  const int D = src.head_dim;
+  const int plane = blockIdx.y;  // (layer of the call, KV head, K / V)
+  const int is_v = plane & 1;
+  const int kvh = (plane >> 1) % src.hkv;
+  const int li = (plane >> 1) / src.hkv;
+  const int layer = layer_begin + li;
+  const int window = layer_window[layer];
+  const int chunks_per_block = 4 * D;  // 64 tokens x D bytes / 16
+  const int64_t B = ci / chunks_per_block;
+  const int x = (int)(ci % chunks_per_block);
+  if (window > 0 && (B + 1) * 64 <= (int64_t)q_pos0 - window + 1) return;
+  const u4 w = load_stream16(cache + src.plane_offset(layer, seq, kvh, is_v) + ci * 16);
+  uint8_t* const out = staged + dst.plane_offset(li, 0, kvh, is_v);
+  const float* const sc = scales + src.scale_offset(layer, seq, is_v, kvh);
+  h8 lo, hi;
+  cvt_i8x16_to_h8x2(w, lo, hi);
+  if (!is_v) {
+    const int tile = x / D, c = (x % D) >> 4, r = x & 15;  // (16-token tile of the block, chunk, row)
+    if (scale_k) {
+      const f4 s0 = *reinterpret_cast<const f4*>(sc + 16 * c), s1 = *reinterpret_cast<const f4*>(sc + 16 * c + 4);
+      const f4 s2 = *reinterpret_cast<const f4*>(sc + 16 * c + 8), s3 = *reinterpret_cast<const f4*>(sc + 16 * c + 12);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = (_Float16)((float)lo[e] * s0[e]);
+        lo[4 + e] = (_Float16)((float)lo[4 + e] * s1[e]);
+        hi[e] = (_Float16)((float)hi[e] * s2[e]);
+        hi[4 + e] = (_Float16)((float)hi[4 + e] * s3[e]);
+      }
+    }
+    uint8_t* t0 = out + (B * 4 + tile) * (int64_t)(32 * D);
+    *reinterpret_cast<h8*>(t0 + ((2 * c) * 16 + r) * 16) = lo;
+    *reinterpret_cast<h8*>(t0 + ((2 * c + 1) * 16 + r) * 16) = hi;
+  } else {
+    const float vs = sc[16 * (x >> 6) + (x & 15)];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      lo[e] = (_Float16)((float)lo[e] * vs);
+      hi[e] = (_Float16)((float)hi[e] * vs);
+    }
+    *reinterpret_cast<h8*>(out + (2 * B) * (int64_t)(64 * D) + x * 16) = lo;
+    *reinterpret_cast<h8*>(out + (2 * B + 1) * (int64_t)(64 * D) + x * 16) = hi;
+  }
+}
+
+// Bytes of the staging area for `n_layers` layers of a call that ends at position `end` (exclusive).
+int64_t prefill_i8_stage_bytes(const CacheGeom& g, int n_layers, int end) {
+  return (int64_t)n_layers * g.hkv * 2 * round_up64(end, kTokenAlign) * g.head_dim * 2;
+}
+
+template <int OUT>
+hipError_t launch_i8(const PrefillArgs& a, PrefillPlans* plans, hipStream_t stream, hipEvent_t ev0, hipEvent_t ev1) {
+  constexpr int D = 256;
+  if (!a.kv_stage || !a.scales || (OUT != kF16 && !a.q_stage)) return hipErrorInvalidValue;
+  const int end = a.q_pos0 + a.n;
+  if (a.kv_stage_bytes < prefill_i8_stage_bytes(a.geom, a.n_layers, end)) return hipErrorInvalidValue;
+  // the staged planes: a half cache of the call's layers and of one sequence, just long enough
+  CacheGeom g = a.geom;
+  g.num_layers = a.n_layers;
+  g.max_seqs = 1;
+  g.cap = (int32_t)round_up64(end, kTokenAlign);
+  g.esize = 2;
+  g.plane_bytes = (int64_t)g.cap * g.head_dim * 2;
+  const int64_t chunks = (int64_t)(g.cap / 64) * 4 * D;
+  // (the first launch of the call carries the start event of a timed call, the attention kernel the stop event)
+  hipExtLaunchKernelGGL(dequant_planes_kernel, dim3((unsigned)((chunks + 255) / 256), a.n_layers * a.geom.hkv * 2), dim3(256),
+                        0, stream, ev0, nullptr, 0, a.cache, a.scales, a.geom, reinterpret_cast<uint8_t*>(a.kv_stage), g,
+                        a.layer_window, a.layer_begin, a.seq, a.q_pos0, chunks, OUT == kF16 ? 1 : 0);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  PrefillArgs b = a;
+  if constexpr (OUT != kF16) {
+    const int64_t pieces = (int64_t)a.n_layers * a.n * a.hq * (D / 8);
+    hipLaunchKernelGGL((stage_queries_i8_kernel<OUT, D>), dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream, a.q,
+                       reinterpret_cast<_Float16*>(a.q_stage), a.scales, a.geom, a.layer_begin, a.seq, a.n, a.hq, a.group,
+                       pieces);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    b.q = a.q_stage;
+  }
+  b.q_staged = 1;
+  b.cache = reinterpret_cast<const uint8_t*>(a.kv_stage);
+  b.geom = g;
+  b.scales = nullptr;
+  b.seq = 0;
+  // (the kernels address layers from layer_begin on; the staged cache starts at the call's first layer)
+  b.layer_begin = 0;
+  b.layer_window = a.layer_window + a.layer_begin;
+  if (a.host_window) b.host_window = a.host_window + a.layer_begin;
+  return launch_typed<kF16, OUT, D>(b, plans, stream, nullptr, ev1);
 }
 
 hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, PrefillPlans* plans, hipStream_t stream,
@@ -1613,6 +1768,9 @@ hipError_t launch_prefill(const PrefillArgs& a, int kv_dtype, int io_dtype, Pref
   if (kv_dtype == kF16 && io_dtype == kF32) return launch_typed<kF16, kF32, 256>(a, plans, stream, ev0, ev1);
   if (kv_dtype == kBF16 && io_dtype == kBF16) return launch_typed<kBF16, kBF16, 256>(a, plans, stream, ev0, ev1);
   if (kv_dtype == kBF16 && io_dtype == kF32) return launch_typed<kBF16, kF32, 256>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kI8 && io_dtype == kF16) return launch_i8<kF16>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kI8 && io_dtype == kBF16) return launch_i8<kBF16>(a, plans, stream, ev0, ev1);
+  if (kv_dtype == kI8 && io_dtype == kF32) return launch_i8<kF32>(a, plans, stream, ev0, ev1);
 #endif
   return hipErrorInvalidValue;
 }
