@@ -108,6 +108,7 @@ struct DecodeArgs {
   int32_t num_splits;
   int32_t max_kv_len;        // max over kv_lens (host computed), sizes the partitions
   int32_t min_kv_len;        // min over kv_lens (host computed; only the launch rules look at it)
+  int32_t rule_batch;        // sequences the launch rules count: batch, or those of the larger batch this launch is a part of
   float scale;               // softmax scale
   float softcap;
   // The step before attention, run by the decode kernel itself for the one new token of every sequence

@@ -721,7 +721,7 @@ hipError_t launch_typed(const DecodeArgs& a, const DecodeTuning& t, hipStream_t 
     // Measured on MI355X (head_dim 256, 4096-token context): with several
     // workgroups per CU one wave each is as fast or faster (fewer LDS merges),
     // with less than one per CU more waves per workgroup hide the latency.
-    const int wgs = a.n_layers * a.batch * a.geom.hkv * a.num_splits;
+    const int wgs = a.n_layers * (a.rule_batch > 0 ? a.rule_batch : a.batch) * a.geom.hkv * a.num_splits;
     waves = wgs >= 768 ? 1 : wgs >= 256 ? 2 : 4;
     // ... and one wave when a partition is one or two key blocks: more waves
     // would only add to the merge (one layer of 1024 tokens in 64-token

@@ -268,9 +268,14 @@ struct NewRows {
 // partials go to this GPU's `scratch` instead of the handle's growable workspace.
 // new_rows: q holds raw query projections and the new token's key / value rows come with the call
 // (its row, kv_lens[b] - 1, need not have been appended).
+// The batch a launch is a part of (mi355_attn_decode_step cuts large batches into several launches): the launch rules
+// then look at the whole batch, so that every part runs as the same sequences would in one launch of all of them,
+// partitions and waves included, and the results are the same bits.
+struct WholeBatch { int batch, max_len, min_len; };
+
 int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq_ids, const int32_t* kv_lens,
                 int batch, const void* q, void* out, int num_splits, char** error_msg, bool no_alloc = false,
-                const NewRows* new_rows = nullptr) {
+                const NewRows* new_rows = nullptr, const WholeBatch* whole = nullptr) {
   if (!h) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null handle");
   if (new_rows) {
     if (!new_rows->k || !new_rows->v) return fail(error_msg, MI355_ATTN_INVALID_ARGUMENT, "null k or v");
@@ -319,12 +324,22 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   HIP_OR_RETURN(hipSetDevice(h->device));
   const int items = n_layers * batch;
   const bool splits_chosen = num_splits == 0;
+  if (whole) {
+    max_len = whole->max_len;
+    min_len = whole->min_len;
+  }
   if (num_splits == 0) {
     // About 1024 workgroups (four waves per CU saturate HBM; measured: 30 layers x 2 KV heads at 4096 tokens
     // run 8 % faster with 16-18 partitions than with 35, 16 layers x 64 sequences fastest without any split),
     // partitions of >= 64 tokens.
-    const int want = (1024 + items * h->cfg.num_kv_heads - 1) / (items * h->cfg.num_kv_heads);
+    const int rule_items = whole ? n_layers * whole->batch : items;
+    const int want = (1024 + rule_items * h->cfg.num_kv_heads - 1) / (rule_items * h->cfg.num_kv_heads);
     num_splits = std::max(1, std::min({want, (max_len + 63) / 64, 64}));
+    // Contexts of up to 512 tokens: one partition, and with it no merge launch. Measured (one layer, fp16, Hq8/Hkv2,
+    // calls queued back to back): 1 sequence of 256 / 512 tokens 6.7 / 8.6 us against 9.9 / 9.8 us split and merged,
+    // 64 sequences 9.7 / 15.4 against 11.0 / 16.1 us, 256 sequences 26.9 / 46.3 against 32.4 / 51.8 us; from 640
+    // tokens on the split wins for small batches (1 sequence of 768 tokens: 10.9 against 9.8 us).
+    if (max_len <= 512) num_splits = 1;
   }
   DecodeArgs a{};
   const size_t slots = (size_t)items * h->cfg.num_q_heads * num_splits;
@@ -403,6 +418,7 @@ int decode_impl(mi355_attn* h, int layer_begin, int n_layers, const int32_t* seq
   a.num_splits = num_splits;
   a.max_kv_len = max_len;
   a.min_kv_len = min_len;
+  a.rule_batch = whole ? whole->batch : batch;
   fill_inline_windows(h, &a);
   bool scratch_fence = false;
   if (no_alloc && num_splits > 1) {
@@ -1003,11 +1019,17 @@ int mi355_attn_decode_step(mi355_attn* h, int32_t layer, const int32_t* seq_ids,
   }
   const size_t q_row = (size_t)h->cfg.num_q_heads * h->cfg.head_dim * io_size(h);
   const size_t kv_row = (size_t)h->cfg.num_kv_heads * h->cfg.head_dim * io_size(h);
+  WholeBatch whole{batch, 0, INT32_MAX};
+  for (int b = 0; b < batch; ++b) {
+    whole.max_len = std::max(whole.max_len, kv_lens[b]);
+    whole.min_len = std::min(whole.min_len, kv_lens[b]);
+  }
   for (int b0 = 0; b0 < batch; b0 += kInlineItems) {
     const int nb = std::min<int>(kInlineItems, batch - b0);
     const NewRows rows{static_cast<const uint8_t*>(k) + b0 * kv_row, static_cast<const uint8_t*>(v) + b0 * kv_row};
     if (int rc = decode_impl(h, layer, 1, ids.data() + b0, kv_lens + b0, nb, static_cast<const uint8_t*>(q) + b0 * q_row,
-                             static_cast<uint8_t*>(out) + b0 * q_row, num_splits, error_msg, /*no_alloc=*/false, &rows))
+                             static_cast<uint8_t*>(out) + b0 * q_row, num_splits, error_msg, /*no_alloc=*/false, &rows,
+                             &whole))
       return rc;
   }
   return MI355_ATTN_OK;

@@ -8,10 +8,12 @@
 // behind the C ABI shape of its GPU sampler plugin
 // (runtime/components/sampler_factory.cc:34-46).
 //
-// Two launches per call. select_kernel: a row of ~262k logits is cut into up to
+// One launch per call (sample_kernel). A row of ~262k logits is cut into up to
 // 16 segments, one workgroup of 1024 threads each, so that one row already
-// spreads over 16 CUs. A workgroup reads its segment once, 16 logits per thread
-// that stay in registers. Every thread takes the maximum of its logits; every
+// spreads over 16 CUs; a call of so many rows that this would make more than two
+// workgroups per compute unit takes segments four times as long. A workgroup
+// reads its segment once, 16 (or 64) logits per thread that stay in registers,
+// all loads issued at once. Every thread takes the maximum of its logits; every
 // wave reports the ceil(k/16)-th largest of its 64 maxima (DPP reductions); at
 // least k logits of the segment reach the smallest of those 16 numbers, so only
 // what reaches it - a few hundred candidates - is packed as (order-preserving
@@ -21,8 +23,11 @@
 // runs of equal values) or that hold fewer than k numbers fall back to a radix
 // descent on the keys with LDS histograms (12 + 12 + 8 bits); exact ties at the
 // k-th value are then taken in ascending index order.
-// finish_kernel: one workgroup per row thresholds and ranks the segments'
-// candidates the same way and walks the k winners in the reference's op order.
+// The workgroup that delivers the last segment of a row (a ticket per row) then
+// thresholds and ranks the segments' candidates the same way and walks the k
+// winners in the reference's op order (finish_row). Vocabularies beyond 16 x
+// 16,384 entries in calls of few rows re-read their segments per pass and run
+// as two launches (select_kernel, finish_kernel).
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <float.h>
@@ -47,8 +52,9 @@ constexpr int kCap = 2048;              // candidates of one segment that fit in
 constexpr int kMaxK = MI355_SAMPLER_MAX_K;
 constexpr int kMaxSegments = 16;
 constexpr int kSlots = kMaxK;            // workspace words per segment; a zero word is an empty slot
-constexpr int kMergeCap = kMaxSegments * kSlots;  // 4096 words of one row in finish_kernel
-constexpr int kResident = 16;           // logits per thread that stay in registers between the passes
+constexpr int kMergeCap = kMaxSegments * kSlots;  // 4096 words of one row in finish_row
+constexpr int kResident = 16;           // logits per thread of a short segment, which stay in registers between the passes
+constexpr int kResidentWide = 64;       // ... and of a wide one (calls with many rows)
 constexpr int kSegmentMin = kThreads * kResident;  // a segment is this long unless the row needs more than kMaxSegments
 
 typedef unsigned long long u64;
@@ -61,6 +67,10 @@ struct SamplerArgs {
   int32_t* topk_idx;      // [batch][k] or null
   float* topk_prob;       // [batch][k] or null
   u64* workspace;         // [batch][segments][kSlots] candidates, (key << 32) | ~index, 0 = empty
+  uint32_t* tickets;      // [batch] segments of the row that are done; all zero between calls (sample_kernel)
+#ifdef MI355_SAMPLER_TRACE
+  unsigned long long* trace;  // [workgroups][16] (event << 56 | 100 MHz time)
+#endif
   int32_t vocab, k, segments, seg_len;
   float p, temperature;
   uint32_t seed;
@@ -228,6 +238,12 @@ __device__ __forceinline__ uint32_t reserve_slots(const u64 (&take)[NV], uint32_
   return (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
 }
 
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every outstanding global load
+// of the wave, and the wide segments' loads are meant to stay in flight across the barrier below.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // The float version (-inf = none): used on the logits themselves.
 __device__ __forceinline__ float lower_bound_of_kth_f32(float v, int k, float* wave_val, int tid) {
   const int lane = tid & 63, wave = tid >> 6;
@@ -239,7 +255,7 @@ __device__ __forceinline__ float lower_bound_of_kth_f32(float v, int k, float* w
     if (lane == __ffsll((long long)holders) - 1) v = -INFINITY;  // drop one holder of the maximum
   }
   if (lane == 0) wave_val[wave] = m;
-  __syncthreads();
+  lds_barrier();
   float tau = wave_val[0];
   for (int w = 1; w < kWavesPerWg; ++w) tau = fminf(tau, wave_val[w]);
   return tau;
@@ -283,25 +299,93 @@ __device__ __forceinline__ void rank_select(const u64* cand, int n, u64* top, in
   }
 }
 
-// The candidates of one segment of one row into the workspace: everything that
+// The candidate workspace is written by one workgroup and read by another of the same launch (sample_kernel),
+// which may sit on another XCD, whose L2 is a different one: stores and loads of device scope, which go
+// through to memory, instead of a write-back and an invalidation of whole caches around ordinary ones (measured:
+// those made the launch three times slower).
+__device__ __forceinline__ void ws_store(u64* p, u64 v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u64 ws_load(const u64* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+#ifdef MI355_SAMPLER_TRACE
+__device__ unsigned long long* g_trace_dev;
+__device__ __forceinline__ void trace_mark(int ev) {
+  __shared__ int n_marks;  // (thread 0 only; set to zero by mark 1)
+  if (threadIdx.x == 0) {
+    if (ev == 1) n_marks = 0;
+    unsigned long long* row = g_trace_dev + (blockIdx.y * gridDim.x + blockIdx.x) * 16;
+    if (n_marks < 16) row[n_marks++] = ((unsigned long long)ev << 56) | (__builtin_amdgcn_s_memrealtime() & 0xffffffffffull);
+  }
+}
+#define TRACE_MARK(ev) trace_mark(ev)
+#else
+#define TRACE_MARK(ev)
+#endif
+
+struct SelectLds {
+  uint32_t hist[kBins];
+  alignas(16) u64 cand[kCap + kRankPad];  // zero behind the last candidate (rank_select)
+  u64 top[kMaxK];
+  uint32_t rank_sm[kThreads];
+  uint32_t wave_sum[kWavesPerWg];
+  uint32_t found[3];  // bin, count above it, count in it
+  uint32_t n_cand, n_ties;
+};
+
+// A segment of up to R logits per thread, read from memory once: it stays in registers for all passes (same
+// index layout as for_each_key); slots past the segment's end hold NaN, which no comparison and no maximum
+// ever picks.
+template <int R>
+__device__ __forceinline__ void load_segment(const SamplerArgs& a, int b, int sgm, float (&xreg)[R]) {
+  const int tid = threadIdx.x;
+  const int index0 = sgm * a.seg_len;
+  const int len = min(a.seg_len, a.vocab - index0);
+  const float* seg = a.logits + (size_t)b * a.vocab + index0;
+  const bool vec_ok = (a.vocab % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
+  if (vec_ok && len == kThreads * R) {
+    // a whole segment (the usual case): all loads at once and nothing between them (behind per-thread
+    // conditions each load would wait for the one before it)
+#pragma unroll
+    for (int u = 0; u < R / 4; ++u) {
+      const float4 x = *reinterpret_cast<const float4*>(seg + u * kPerIter + tid * 4);
+      xreg[4 * u] = x.x; xreg[4 * u + 1] = x.y; xreg[4 * u + 2] = x.z; xreg[4 * u + 3] = x.w;
+    }
+    return;
+  }
+#pragma unroll
+  for (int u = 0; u < R / 4; ++u) {
+    const int base = u * kPerIter + tid * 4;
+    if (vec_ok && base + 3 < len) {
+      const float4 x = *reinterpret_cast<const float4*>(seg + base);
+      xreg[4 * u] = x.x; xreg[4 * u + 1] = x.y; xreg[4 * u + 2] = x.z; xreg[4 * u + 3] = x.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xreg[4 * u + j] = base + j < len ? seg[base + j] : __int_as_float(0x7fc00000);
+    }
+  }
+}
+
+// The candidates of segment `sgm` of row `b` into the workspace: everything that
 // reaches the threshold when that is at most kSlots words (the usual case: the
 // row's kernel ranks them anyway), else the segment's k largest.
-// RESIDENT: every segment has at most kSegmentMin logits (the host knows), which
-// then stay in registers; the other instantiation re-reads them (from L2) per pass.
-// 64 registers at most, so that two workgroups share a compute unit.
-template <bool RESIDENT>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
-select_kernel(const SamplerArgs a) {
-  __shared__ uint32_t hist[kBins];
-  __shared__ __align__(16) u64 cand[kCap + kRankPad];  // zero behind the last candidate (rank_select)
-  __shared__ u64 top[kMaxK];
-  __shared__ uint32_t rank_sm[kThreads];
-  __shared__ uint32_t wave_sum[kWavesPerWg];
-  __shared__ uint32_t found[3];  // bin, count above it, count in it
-  __shared__ uint32_t n_cand, n_ties;
+// R > 0: the segment has at most kThreads * R logits (the host knows) and xreg holds them (load_segment);
+// R == 0: they are re-read (from L2) per pass, xreg is unused. Every return is taken by the whole workgroup.
+template <int R>
+__device__ __forceinline__ void select_segment(const SamplerArgs& a, SelectLds& sm, int b, int sgm,
+                                               const float (&xreg)[R > 0 ? R : 1]) {
+  uint32_t* const hist = sm.hist;
+  u64* const cand = sm.cand;
+  u64* const top = sm.top;
+  uint32_t* const rank_sm = sm.rank_sm;
+  uint32_t* const wave_sum = sm.wave_sum;
+  uint32_t* const found = sm.found;
+  uint32_t& n_cand = sm.n_cand;
+  uint32_t& n_ties = sm.n_ties;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int b = blockIdx.y, sgm = blockIdx.x;
   const int index0 = sgm * a.seg_len;                 // first vocabulary index of the segment
   const int len = min(a.seg_len, a.vocab - index0);   // > 0 by construction of the grid
   const int k = min(a.k, len);
@@ -309,28 +393,13 @@ select_kernel(const SamplerArgs a) {
   const bool vec_ok = (a.vocab % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
   u64* out = a.workspace + ((size_t)b * a.segments + sgm) * kSlots;
 
-  // A segment of up to 16 logits per thread is read from memory once and stays in
-  // registers for all later passes (same index layout as for_each_key); slots past
-  // the segment's end hold NaN, which no comparison and no maximum ever picks.
-  constexpr bool resident = RESIDENT;
-  float xreg[RESIDENT ? kResident : 1];
-  if constexpr (resident) {
-#pragma unroll
-    for (int u = 0; u < kResident / 4; ++u) {
-      const int base = u * kPerIter + tid * 4;
-      if (vec_ok && base + 3 < len) {
-        const float4 x = *reinterpret_cast<const float4*>(seg + base);
-        xreg[4 * u] = x.x; xreg[4 * u + 1] = x.y; xreg[4 * u + 2] = x.z; xreg[4 * u + 3] = x.w;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xreg[4 * u + j] = base + j < len ? seg[base + j] : __int_as_float(0x7fc00000);
-      }
-    }
-  }
+  constexpr bool resident = R > 0;
+  // (the passes of the rare paths below go over the registers of a short segment, but re-read a wide one, from
+  // L2: unrolled over 64 registers they would be most of the kernel's code and cost the common path registers)
   auto each = [&](auto&& f) {
-    if constexpr (resident) {
+    if constexpr (resident && R <= kResident) {
 #pragma unroll
-      for (int u = 0; u < kResident / 4; ++u)
+      for (int u = 0; u < R / 4; ++u)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int i = u * kPerIter + tid * 4 + j;
@@ -351,9 +420,9 @@ select_kernel(const SamplerArgs a) {
     __syncthreads();
     if (tid == 0) {
       for (int w = 1; w < kWavesPerWg; ++w) best = max(best, cand[w]);
-      out[0] = best;
+      ws_store(out, best);
     }
-    for (int i = 1 + tid; i < kSlots; i += kThreads) out[i] = 0;
+    for (int i = 1 + tid; i < kSlots; i += kThreads) ws_store(out + i, 0);
     return;
   }
 
@@ -364,24 +433,27 @@ select_kernel(const SamplerArgs a) {
     // on the logits themselves: three instructions per logit, keys only for the candidates
     float tmax = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < kResident; ++e) tmax = fmaxf(tmax, xreg[e]);
+    for (int e = 0; e < R; ++e) tmax = fmaxf(tmax, xreg[e]);
     if (tid == 0) n_cand = 0;
     const float tau = lower_bound_of_kth_f32(tmax, k, reinterpret_cast<float*>(wave_sum), tid);  // (barrier inside)
-    u64 take[kResident];
+    TRACE_MARK(6);
+    // sixteen logits per thread at a time (their ballots live in scalar registers)
 #pragma unroll
-    for (int e = 0; e < kResident; ++e) take[e] = __ballot(xreg[e] >= tau);
-    uint32_t slot0 = reserve_slots(take, &n_cand, lane);
+    for (int c0 = 0; c0 < R; c0 += 16) {
+      u64 take[16];
 #pragma unroll
-    for (int u = 0; u < kResident / 4; ++u)
+      for (int e = 0; e < 16; ++e) take[e] = __ballot(xreg[c0 + e] >= tau);
+      uint32_t slot0 = reserve_slots(take, &n_cand, lane);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int e = 4 * u + j;
+      for (int e = 0; e < 16; ++e) {
         if (take[e]) {  // (uniform over the wave; most are zero)
           const uint32_t pos = slot0 + lanes_below(take[e]);
-          if (xreg[e] >= tau && pos < (uint32_t)kCap) cand[pos] = pack(key_of(xreg[e]), index0 + u * kPerIter + tid * 4 + j);
+          const int u = (c0 + e) >> 2, j = (c0 + e) & 3;
+          if (xreg[c0 + e] >= tau && pos < (uint32_t)kCap) cand[pos] = pack(key_of(xreg[c0 + e]), index0 + u * kPerIter + tid * 4 + j);
           slot0 += (uint32_t)__popcll(take[e]);
         }
       }
+    }
     __syncthreads();
   } else {
     uint32_t tmax = 0;
@@ -399,11 +471,12 @@ select_kernel(const SamplerArgs a) {
     });
     __syncthreads();
   }
+  TRACE_MARK(7);
   // (n_cand is only written again behind further barriers)
   const bool fast_ok = n_cand <= (uint32_t)kCap && n_cand >= (uint32_t)k;  // (fewer than k: NaNs among the logits)
   if (fast_ok && n_cand <= (uint32_t)kSlots) {
     const int n = (int)n_cand;
-    if (tid < kSlots) out[tid] = tid < n ? cand[tid] : 0;
+    if (tid < kSlots) ws_store(out + tid, tid < n ? cand[tid] : 0);
     return;
   }
 
@@ -477,43 +550,72 @@ select_kernel(const SamplerArgs a) {
   }
   const int n = (int)n_cand;  // k <= n <= kCap
   rank_select(cand, n, top, k, rank_sm, tid);
-  if (tid < kSlots) out[tid] = tid < k ? top[tid] : 0;
+  if (tid < kSlots) ws_store(out + tid, tid < k ? top[tid] : 0);
 }
 
-// Merges the segments' candidates of one row and draws (sampling_cpu_util.cc:98-131, 189-230).
-__global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
-  __shared__ __align__(16) u64 surv[kMergeCap + kRankPad];  // the segments' candidates that reach the threshold, then zeros
-  __shared__ u64 cand[kMaxK];      // the row's k winners, descending
-  __shared__ __align__(16) float e_sm[kMaxK + 16];  // (+16: the loops below read up to 15 entries past the last one they use)
-  __shared__ uint32_t rank_sm[kThreads];
-  __shared__ uint32_t wave_val[kWavesPerWg];
-  __shared__ uint32_t n_surv;
-  __shared__ float inv_sm;
-  __shared__ double cum_sm[kMaxK];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, b = blockIdx.x;
+// Grid (segments, rows): the first of two launches for rows whose segments do not fit in registers.
+// 64 registers at most, so that two workgroups share a compute unit.
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8)))
+select_kernel(const SamplerArgs a) {
+  __shared__ SelectLds sm;
+  const float none[1] = {0.f};
+  select_segment<0>(a, sm, blockIdx.y, blockIdx.x, none);
+}
+
+struct FinishLds {
+  alignas(16) u64 surv[kMergeCap + kRankPad];  // the segments' candidates that reach the threshold, then zeros
+  u64 cand[kMaxK];      // the row's k winners, descending
+  alignas(16) float e_sm[kMaxK + 16];  // (+16: the loops below read up to 15 entries past the last one they use)
+  uint32_t rank_sm[kThreads];
+  uint32_t wave_val[kWavesPerWg];
+  uint32_t n_surv;
+  float inv_sm;
+  double cum_sm[kMaxK];
+};
+
+// Merges the segments' candidates of row `b` and draws (sampling_cpu_util.cc:98-131, 189-230). Returns early
+// for the waves that hold none of the k winners: the caller has nothing left to do after it but for thread 0.
+__device__ __forceinline__ void finish_row(const SamplerArgs& a, FinishLds& sm, int b) {
+  u64* const surv = sm.surv;
+  u64* const cand = sm.cand;
+  float* const e_sm = sm.e_sm;
+  uint32_t* const rank_sm = sm.rank_sm;
+  uint32_t* const wave_val = sm.wave_val;
+  uint32_t& n_surv = sm.n_surv;
+  float& inv_sm = sm.inv_sm;
+  double* const cum_sm = sm.cum_sm;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int k = min(a.k, a.vocab);
-  // Wave s holds the kSlots words of segment s, four consecutive ones per thread;
-  // zero words are empty slots (a segment fills its slots from the front).
+  // The row's n = segments x kSlots words (zero words are empty slots; a segment fills its slots from the front).
+  // More than four segments: wave s holds the words of segment s, four consecutive ones per thread. Up to four:
+  // one word per thread, every fourth slot of a segment per wave, so that each of the 4 x segments waves gets its
+  // share of the filled slots at the front (the bound below takes a wave with few words for an empty one).
   const int n = a.segments * kSlots;  // <= kMergeCap
   const u64* in = a.workspace + (size_t)b * n;
-  u64 w[4];
+  const bool one_each = n <= kThreads;
+  const int waves = one_each ? n / 64 : n / 256;
+  u64 w[4] = {0, 0, 0, 0};
   uint32_t wmax = 0;
-  if (4 * tid < n) {
-    const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(in + 4 * tid);
-    const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(in + 4 * tid + 2);
-    w[0] = lo.x; w[1] = lo.y; w[2] = hi.x; w[3] = hi.y;
-  } else {
-    w[0] = w[1] = w[2] = w[3] = 0;
+  static_assert(kSlots == 4 * 64, "one wave of four-word threads per segment, or four waves of one-word threads");
+  if (one_each) {
+    if (tid < n) {
+      const int r = tid % kSlots;
+      w[0] = ws_load(in + (tid - r) + (r % 64) * 4 + r / 64);
+    }
+  } else if (4 * tid < n) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = ws_load(in + 4 * tid + j);
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) wmax = max(wmax, (uint32_t)(w[j] >> 32));
   if (tid == 0) n_surv = 0;
   rank_sm[tid] = 0;  // (for rank_select)
   for (int i = tid; i < kMergeCap + kRankPad; i += kThreads) surv[i] = 0;
-  // same scheme as in select_kernel: a lower bound of the k-th largest key, the
+  // same scheme as in select_segment: a lower bound of the k-th largest key, the
   // words that reach it, their ranks by counting
-  static_assert(kSlots == 4 * 64, "one wave of four-word threads per segment");
-  const uint32_t tau = lower_bound_of_kth(wmax, k, a.segments, wave_val, tid);  // (barrier inside)
+  TRACE_MARK(8);
+  const uint32_t tau = lower_bound_of_kth(wmax, k, waves, wave_val, tid);  // (barrier inside)
+  TRACE_MARK(9);
   u64 take[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) take[j] = __ballot(w[j] != 0 && (uint32_t)(w[j] >> 32) >= tau);
@@ -524,11 +626,12 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
     slot0 += (uint32_t)__popcll(take[j]);
   }
   __syncthreads();
+  TRACE_MARK(10);
   rank_select(surv, (int)n_surv, cand, k, rank_sm, tid);
-  // The rest is the work of k threads: the other waves leave (a barrier waits
-  // only for the waves of the workgroup that are still running).
+  TRACE_MARK(11);
+  // The rest is the work of k threads: the other waves leave (a barrier waits only for the waves of the workgroup
+  // that are still running; nothing comes after the merge for them in either kernel).
   if (tid >= ((k + 63) & ~63)) return;
-
   if (k == 1) {
     if (tid == 0) {
       const int idx = index_of(cand[0]);
@@ -589,10 +692,11 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
     reaches = c >= (double)a.p;
   }
   // the first thread of all that reaches p (k - 1 if none does: then the nucleus is all k candidates)
-  const int k_waves = (k + 63) >> 6;  // the waves that are still here
+  const int k_waves = (k + 63) >> 6;  // the waves that hold winners
+  static_assert(kMaxK <= 8 * 64, "wave_val holds two entries per wave of winners");
   {
     const u64 m = __ballot(reaches);
-    if (lane == 0) wave_val[wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
+    if (lane == 0 && wave < k_waves) wave_val[wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
   }
   __syncthreads();
   int first_reach = k - 1;
@@ -606,7 +710,7 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
   const double draw = (double)u01 * mass;
   {
     const u64 m = __ballot(tid < nucleus && draw <= cum_sm[tid]);
-    if (lane == 0) wave_val[8 + wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
+    if (lane == 0 && wave < k_waves) wave_val[8 + wave] = m ? (uint32_t)(wave * 64 + __ffsll((long long)m) - 1) : (uint32_t)kMaxK;
   }
   __syncthreads();
   if (tid == 0) {
@@ -621,6 +725,57 @@ __global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
     if (a.topk_idx) a.topk_idx[(size_t)b * k + tid] = index_of(cand[tid]);
     if (a.topk_prob) a.topk_prob[(size_t)b * k + tid] = e_sm[tid];
   }
+}
+
+// Grid (rows): the second of the two launches.
+__global__ void __launch_bounds__(kThreads) finish_kernel(const SamplerArgs a) {
+  __shared__ FinishLds sm;
+  finish_row(a, sm, blockIdx.x);
+}
+
+// Both steps in one launch, for rows whose segments stay in registers: grid (segments, rows), one workgroup per
+// segment of R logits per thread. Every load of the segment is issued at once, so that the whole call is on its
+// way from HBM from the first microsecond on; the per-thread maxima are taken as the loads land. The workgroup
+// that delivers the last segment of a row (a ticket per row, drawn once the segment's candidates are written)
+// finishes the row.
+template <int R>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(R <= kResident ? 8 : 4, R <= kResident ? 8 : 4)))
+sample_kernel(const SamplerArgs a) {
+  __shared__ union Lds {
+    SelectLds select;
+    FinishLds finish;
+    __device__ Lds() {}
+  } sm;
+  __shared__ uint32_t ticket_sm;
+  const int tid = threadIdx.x;
+  const int b = blockIdx.y, sgm = blockIdx.x;
+#ifdef MI355_SAMPLER_TRACE
+  int n_ev = 0;
+  auto mark = [&](int ev) { (void)n_ev; trace_mark(ev); };
+#else
+  auto mark = [&](int) {};
+#endif
+  mark(1);
+  float xreg[R];
+  load_segment<R>(a, b, sgm, xreg);
+#ifdef MI355_SAMPLER_TRACE
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  mark(2);
+#endif
+  select_segment<R>(a, sm.select, b, sgm, xreg);
+  mark(3);
+  // The candidates are written (ws_store): once every thread's stores have been acknowledged, draw the row's
+  // ticket. Who draws the last one reads what the others wrote before they drew theirs (ws_load).
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  if (tid == 0) ticket_sm = __hip_atomic_fetch_add(a.tickets + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  mark(4);
+  if (ticket_sm != (uint32_t)a.segments - 1u) return;
+  __syncthreads();  // (the arrays of the selection become those of the merge)
+  finish_row(a, sm.finish, b);
+  mark(5);
+  if (tid == 0) a.tickets[b] = 0;  // for the next launch
 }
 
 int fail(char** error_msg, int code, const char* fmt, ...) {
@@ -646,6 +801,13 @@ int fail(char** error_msg, int code, const char* fmt, ...) {
 
 }  // namespace
 
+#ifdef MI355_SAMPLER_TRACE  // (development builds: a timeline per workgroup)
+static unsigned long long* g_trace = nullptr;
+extern "C" int mi355_sampler_trace_read(void* dst, size_t bytes) {
+  return (int)hipMemcpy(dst, g_trace, bytes, hipMemcpyDeviceToHost);
+}
+#endif
+
 struct mi355_sampler {
   mi355_sampler_config cfg{};
   int k = 1;
@@ -664,7 +826,9 @@ struct mi355_sampler {
   float* d_topk_prob = nullptr;
   // candidates of the segments, [batch][segments][k]
   unsigned long long* d_workspace = nullptr;
+  uint32_t* d_tickets = nullptr;  // [batch], all zero between calls
   int segments = 1, seg_len = 0;
+  bool wide = false;  // segments of up to kThreads * kResidentWide logits (sample_kernel<kResidentWide>)
 };
 
 namespace {
@@ -700,17 +864,28 @@ int run(mi355_sampler* h, const float* logits, const float* uniforms, int32_t* i
   a.workspace = h->d_workspace;
   a.segments = h->segments;
   a.seg_len = h->seg_len;
-  // ev0 / ev1 ride on the dispatches: begin of the first kernel, end of the second
-  if (h->seg_len <= kSegmentMin)
-    hipExtLaunchKernelGGL(select_kernel<true>, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
-                          h->timing ? h->ev0 : nullptr, nullptr, 0, a);
-  else
-    hipExtLaunchKernelGGL(select_kernel<false>, dim3((unsigned)h->segments, (unsigned)B), dim3(kThreads), 0, h->stream,
-                          h->timing ? h->ev0 : nullptr, nullptr, 0, a);
-  HIP_OR_RETURN(hipGetLastError());
-  hipExtLaunchKernelGGL(finish_kernel, dim3((unsigned)B), dim3(kThreads), 0, h->stream, nullptr,
-                        h->timing ? h->ev1 : nullptr, 0, a);
-  HIP_OR_RETURN(hipGetLastError());
+  a.tickets = h->d_tickets;
+#ifdef MI355_SAMPLER_TRACE
+  if (!g_trace) HIP_OR_RETURN(hipMalloc(&g_trace, 8 * 16 * 4096));
+  HIP_OR_RETURN(hipMemsetAsync(g_trace, 0, 8 * 16 * 4096, h->stream));
+  a.trace = g_trace;
+  HIP_OR_RETURN(hipMemcpyToSymbol(HIP_SYMBOL(g_trace_dev), &g_trace, sizeof(g_trace)));
+#endif
+  // ev0 / ev1 ride on the dispatches: begin of the first kernel, end of the last
+  hipEvent_t e0 = h->timing ? h->ev0 : nullptr, e1 = h->timing ? h->ev1 : nullptr;
+  const dim3 grid((unsigned)h->segments, (unsigned)B);
+  if (h->seg_len <= kSegmentMin) {
+    hipExtLaunchKernelGGL(sample_kernel<kResident>, grid, dim3(kThreads), 0, h->stream, e0, e1, 0, a);
+    HIP_OR_RETURN(hipGetLastError());
+  } else if (h->wide) {
+    hipExtLaunchKernelGGL(sample_kernel<kResidentWide>, grid, dim3(kThreads), 0, h->stream, e0, e1, 0, a);
+    HIP_OR_RETURN(hipGetLastError());
+  } else {
+    hipExtLaunchKernelGGL(select_kernel, grid, dim3(kThreads), 0, h->stream, e0, nullptr, 0, a);
+    HIP_OR_RETURN(hipGetLastError());
+    hipExtLaunchKernelGGL(finish_kernel, dim3((unsigned)B), dim3(kThreads), 0, h->stream, nullptr, e1, 0, a);
+    HIP_OR_RETURN(hipGetLastError());
+  }
   h->timed = h->timing;
   if (h->cfg.host_io) {
     if (ids) HIP_OR_RETURN(hipMemcpyAsync(ids, h->d_ids, B * sizeof(int32_t), hipMemcpyDeviceToHost, h->stream));
@@ -776,14 +951,27 @@ int mi355_sampler_create(const mi355_sampler_config* c, mi355_sampler** out, cha
   }
   if ((e = hipEventCreate(&h->ev0)) != hipSuccess || (e = hipEventCreate(&h->ev1)) != hipSuccess)
     return bail(MI355_SAMPLER_INTERNAL, "hipEventCreate", e);
-  // segments of kSegmentMin logits or less (a multiple of 4), unless that would take more than kMaxSegments
-  // 1, 2, 4, 8 or 16 segments (with three, the row's kernel could not bound its candidates: lower_bound_of_kth)
+  // Segments of kSegmentMin logits or less (a multiple of 4), unless that would take more than kMaxSegments:
+  // 1, 2, 4, 8 or 16 segments (with three, the row's kernel could not bound its candidates: lower_bound_of_kth).
+  // A call of so many rows that the short segments would make more than two workgroups per compute unit takes
+  // segments four times as long (64 logits per thread in registers): the threshold, the barriers and the ticket
+  // are then paid once for four times the logits, and the row's merge has a quarter of the words to look at.
   h->segments = 1;
   while (h->segments < kMaxSegments && (size_t)h->segments * kSegmentMin < (size_t)c->vocab_size) h->segments *= 2;
+  if (h->segments >= 4 && (size_t)c->batch_size * h->segments > 2 * (size_t)std::max(1, prop.multiProcessorCount) &&
+      (size_t)(h->segments / 4) * kThreads * kResidentWide >= (size_t)c->vocab_size) {
+    h->segments /= 4;
+    h->wide = true;
+  }
   h->seg_len = ((c->vocab_size + h->segments - 1) / h->segments + 3) / 4 * 4;
   h->segments = (c->vocab_size + h->seg_len - 1) / h->seg_len;
   if ((e = hipMalloc(&h->d_workspace, sizeof(unsigned long long) * c->batch_size * h->segments * kSlots)) != hipSuccess)
     return bail(MI355_SAMPLER_RESOURCE_EXHAUSTED, "candidate workspace", e);
+  if ((e = hipMalloc(&h->d_tickets, sizeof(uint32_t) * c->batch_size)) != hipSuccess)
+    return bail(MI355_SAMPLER_RESOURCE_EXHAUSTED, "row tickets", e);
+  if ((e = hipMemsetAsync(h->d_tickets, 0, sizeof(uint32_t) * c->batch_size, h->stream)) != hipSuccess ||
+      (e = hipStreamSynchronize(h->stream)) != hipSuccess)
+    return bail(MI355_SAMPLER_INTERNAL, "row tickets clear", e);
   if (c->host_io) {
     const size_t B = c->batch_size, V = c->vocab_size, K = std::min<size_t>(k, V);
     if ((e = hipMalloc(&h->d_logits, B * V * sizeof(float))) != hipSuccess ||
@@ -803,7 +991,7 @@ void mi355_sampler_destroy(mi355_sampler* h) {
   (void)hipSetDevice(h->cfg.device);
   (void)hipStreamSynchronize(h->stream);
   for (void* p : {(void*)h->d_logits, (void*)h->d_uniforms, (void*)h->d_ids, (void*)h->d_scores, (void*)h->d_topk_idx,
-                  (void*)h->d_topk_prob, (void*)h->d_workspace})
+                  (void*)h->d_topk_prob, (void*)h->d_workspace, (void*)h->d_tickets})
     if (p) (void)hipFree(p);
   if (h->ev0) (void)hipEventDestroy(h->ev0);
   if (h->ev1) (void)hipEventDestroy(h->ev1);

@@ -204,3 +204,35 @@ def test_host_io_and_large_batch():
     want, want_sc = so.top_k_top_p_sample(logits, 64, 0.95, 1.0, u)
     assert ids.tolist() == want.tolist()
     np.testing.assert_allclose(sc, so.log_scores(want_sc), rtol=1e-5, atol=1e-6)
+
+
+# Calls of many rows: segments four times as long (64 logits per thread in registers, sample_kernel<64>), chosen when
+# rows x 16,384-logit segments would be more than two workgroups per compute unit.
+@pytest.mark.parametrize("vocab,k,b", [(262144, 64, 40), (262144, 256, 33), (250001, 50, 48), (131072, 1, 80),
+                                       (70000, 17, 160)])
+def test_many_rows_take_wide_segments_and_match_oracle(vocab, k, b):
+    rng = np.random.default_rng(vocab + k + b)
+    logits = (rng.standard_normal((b, vocab)) * 4).astype(np.float32)
+    logits[1, ::3] = logits[1, 0]          # long runs of equal values: the radix descent
+    logits[2] = np.round(logits[2])        # heavy ties at the top
+    logits[3, : vocab // 2] = -np.inf
+    logits[4, 5::7] = np.nan               # NaNs never win
+    logits[5] = 1.5                        # every logit equal: ties in ascending index order
+    logits[6, : vocab - 3] = -np.inf       # fewer than k finite values (k > 3)
+    idx, pr = top_k(logits, k, 0.8)
+    want_idx = so.top_k_indices(logits, k)
+    assert np.array_equal(idx, want_idx), (vocab, k, b, np.argwhere((idx != want_idx).any(axis=1)).ravel()[:8])
+    want_pr, _ = so.softmax_top_k(logits, want_idx, 0.8)
+    np.testing.assert_allclose(pr, want_pr, rtol=2e-6, atol=1e-30)
+    # and a draw with given uniforms, twice on the same sampler (the rows' tickets must be back at zero)
+    u = rng.random(b).astype(np.float32)
+    with S.Sampler(k, 0.9, 0.8, b, 1, vocab, stream=torch.cuda.current_stream().cuda_stream) as s:
+        lg = torch.from_numpy(logits).to(DEV)
+        ud = torch.from_numpy(u).to(DEV)
+        want, _ = so.top_k_top_p_sample(logits, k, 0.9, 0.8, u)
+        for _ in range(3):
+            ids = torch.full((b,), -1, dtype=torch.int32, device=DEV)
+            s.sample_to_id_and_score_buffer(lg, ids, None, ud)
+            torch.cuda.synchronize()
+            assert ids.cpu().numpy().tolist() == want.tolist()
+    say(f"sampler wide segments vocab={vocab} k={k} rows={b}: ok")
