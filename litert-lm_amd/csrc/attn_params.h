@@ -147,6 +147,7 @@ struct PrefillArgs {
   void* q_stage;   // room for the call's queries in the type the matrix cores take, 2 bytes per element, where that is
                    // not the activations' type: float32 activations, bfloat16 activations over an int8 cache
   int32_t q_staged;        // != 0: q is of the kernels' type already (set by the int8 path for the kernels it runs)
+  int32_t plan_layer_offset;  // added to layer_begin in the key of the plan cache (launches over staged planes)
   void* kv_stage;          // int8 cache: room for the half planes the call reads (prefill_i8_stage_bytes)
   int64_t kv_stage_bytes;
   const uint8_t* cache;

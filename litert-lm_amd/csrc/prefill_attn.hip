@@ -1354,7 +1354,9 @@ void release_plan_slot(PrefillPlans* p, int s) {
 // that needs no plan.
 hipError_t plan_for(const PrefillArgs& a, int hpb, int wgs, int cus, PrefillPlans* p, hipStream_t stream, int* slot_out) {
   *slot_out = -1;
-  const int64_t key[8] = {a.layer_begin, a.n_layers, a.q_pos0, a.n, a.kchunk, wgs, hpb, a.seq};
+  // (layer_begin + plan_layer_offset: the first layer of the handle that the launch covers, whose windows the plan
+  // depends on; a launch over staged planes addresses its layers from 0)
+  const int64_t key[8] = {a.layer_begin + a.plan_layer_offset, a.n_layers, a.q_pos0, a.n, a.kchunk, wgs, hpb, a.seq};
   for (int s = 0; s < PrefillPlans::kSlots; ++s)
     if (p->valid[s] && std::equal(key, key + 8, p->key[s])) {
       p->last_use[s] = ++p->clock;
@@ -1754,6 +1756,7 @@ hipError_t launch_i8(const PrefillArgs& a, PrefillPlans* plans, hipStream_t stre
   b.seq = 0;
   // (the kernels address layers from layer_begin on; the staged cache starts at the call's first layer)
   b.layer_begin = 0;
+  b.plan_layer_offset = a.layer_begin;
   b.layer_window = a.layer_window + a.layer_begin;
   if (a.host_window) b.host_window = a.host_window + a.layer_begin;
   return launch_typed<kF16, OUT, D>(b, plans, stream, nullptr, ev1);

@@ -221,3 +221,23 @@ def test_recorded_into_a_graph_without_room_it_takes_the_rowwise_path():
             eager = prefill(at, 0, 0, 0, qd, rowwise=True)
             assert torch.equal(out, eager)
             del g
+
+
+def test_passes_with_different_windows_do_not_share_a_work_plan():
+    # two passes of four layers each through the planned kernel: global layers first, then narrow windows. The
+    # passes' launches have the same shape (layers counted from the staged planes' first), so the plan cache must
+    # tell them apart by the handle's layer they start at.
+    L, hq, hkv, n = 512, 8, 2, 512
+    windows = [0, 0, 0, 0, 40, 40, 40, 40]
+    with make(8, hq, hkv, L, 1, A.F16, layer_window=windows) as at:
+        kv = [fill_int8(at, layer, 0, gen(140 + layer, L, hkv, D), gen(150 + layer, L, hkv, D)) for layer in range(8)]
+        qd, qr = queries(gen(160, 8, n, hq, D), A.F16)
+        at.set_option("prefill_rows16", 1)
+        at.set_option("prefill_key_split", 4)  # (tiles of the global layers in up to four parts, the windowed ones whole)
+        at.set_option("prefill_i8_stage_mib", 4)
+        for _ in range(2):  # (the second call finds both plans cached)
+            out = prefill(at, 0, 0, 0, qd, n_layers=8).float().cpu().numpy()
+            for layer in range(8):
+                ref = c_oracle.sdpa_f64(qr[layer], kv[layer][0], kv[layer][1], D ** -0.5, q_pos0=0,
+                                        window=windows[layer], kv_len=n)
+                assert plain_err(out[layer], ref) < TOL, layer
